@@ -1,0 +1,262 @@
+/*
+ * ttmi.h -- C ABI of libttmi.so, the MI355X (gfx950 / CDNA4) device layer behind the
+ * TurboTransformers BERT encoder-layer hot path.
+ *
+ * Every entry point takes plain pointers, sizes and enums; nothing from HIP, torch or
+ * pybind11 appears in a signature, so host C++ (or any FFI) can bind it without HIP
+ * headers.  It replaces the `#ifdef TT_WITH_CUDA` device branches of the reference's
+ * kernel and core layers; each declaration cites the reference interface it stands in
+ * for (paths relative to the reference tree).
+ *
+ * Conventions
+ *   - all tensors are dense row-major unless a leading dimension is given;
+ *   - `dtype` selects the storage type of activations/weights (TTMI_F32 / F16 / BF16);
+ *     reductions, softmax, LayerNorm and GEMM accumulation are always fp32
+ *     (int32 for TTMI_I8 GEMMs);
+ *   - `stream` is a `hipStream_t` passed as `void*` (NULL = the legacy default stream);
+ *     kernels are enqueued and NOT synchronised;
+ *   - every function returns 0 on success or a negative TTMI_E* code, and
+ *     ttmi_last_error() then returns a thread-local message.
+ */
+#ifndef TTMI_H_
+#define TTMI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTMI_API __attribute__((visibility("default")))
+
+enum ttmi_dtype { TTMI_F32 = 0, TTMI_F16 = 1, TTMI_BF16 = 2, TTMI_I8 = 3, TTMI_I32 = 4, TTMI_I64 = 5 };
+enum ttmi_act { TTMI_ACT_GELU = 0, TTMI_ACT_TANH = 1, TTMI_ACT_RELU = 2 };
+enum ttmi_memcpy_kind { TTMI_H2D = 0, TTMI_D2H = 1, TTMI_D2D = 2 };
+enum ttmi_status {
+  TTMI_OK = 0,
+  TTMI_EINVAL = -1,      /* bad argument / unsupported shape */
+  TTMI_EDEVICE = -2,     /* a HIP runtime call failed */
+  TTMI_ENOMEM = -3,      /* hipMalloc failed */
+  TTMI_EINDEX = -4       /* an embedding id was out of range (reported by ttmi_check_async) */
+};
+
+/* Epilogues a GEMM can apply to its fp32 accumulators before the single store to HBM. */
+enum ttmi_epilogue {
+  TTMI_EPI_NONE = 0,          /* C = alpha*acc + beta*C                                   */
+  TTMI_EPI_BIAS = 1,          /* C = acc + bias[n]                                        */
+  TTMI_EPI_BIAS_ACT = 2,      /* C = act(acc + bias[n])             (AddBiasAct fused)    */
+  TTMI_EPI_BIAS_RESIDUAL = 3, /* C = acc + bias[n] + residual[m,n]  (pre-LayerNorm sum)   */
+  TTMI_EPI_QKV_SPLIT = 4,     /* acc + bias -> q,k,v [B,h,S,d]      (SplitAddBiasTranspose fused) */
+  TTMI_EPI_QKV_SPLIT_PAD = 5  /* packed rows -> zero-padded q,k,v [B,h,maxS,d]            */
+};
+
+/* ------------------------------------------------------------------ runtime ---------- */
+
+TTMI_API const char* ttmi_last_error(void);
+
+/* Device bring-up and properties.  Replaces core::CUDADeviceContext
+ * (turbo_transformers/core/cuda_device_context.cpp:23-46). */
+TTMI_API int ttmi_device_count(int* count);
+TTMI_API int ttmi_set_device(int device);
+TTMI_API int ttmi_device_info(char* name, int name_len, int* compute_units, int* clock_khz,
+                              int64_t* hbm_bytes, int* lds_bytes_per_cu);
+TTMI_API int ttmi_mem_info(int64_t* free_bytes, int64_t* total_bytes);
+
+/* Raw device memory.  Replaces allocator_impl.cpp's cudaMalloc/cudaFree branch
+ * (turbo_transformers/core/allocator/allocator_impl.cpp:20-56). */
+TTMI_API int ttmi_malloc(void** ptr, size_t bytes);
+TTMI_API int ttmi_free(void* ptr);
+/* Pinned host memory for staging copies. */
+TTMI_API int ttmi_host_malloc(void** ptr, size_t bytes);
+TTMI_API int ttmi_host_free(void* ptr);
+
+/* Copies.  `ttmi_memcpy` is synchronous with respect to the host like core::Memcpy
+ * (turbo_transformers/core/memory.cpp:34-81): it is enqueued on `stream` and the stream
+ * is then synchronised.  `ttmi_memcpy_async` only enqueues. */
+TTMI_API int ttmi_memcpy(void* dst, const void* src, size_t bytes, int kind, void* stream);
+TTMI_API int ttmi_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* stream);
+TTMI_API int ttmi_memset_zero(void* dst, size_t bytes, void* stream); /* fill kernel, graph-safe */
+
+TTMI_API int ttmi_stream_create(void** stream);
+TTMI_API int ttmi_stream_destroy(void* stream);
+TTMI_API int ttmi_stream_sync(void* stream);
+TTMI_API int ttmi_event_create(void** event);
+TTMI_API int ttmi_event_destroy(void* event);
+TTMI_API int ttmi_event_record(void* event, void* stream);
+TTMI_API int ttmi_event_sync(void* event);
+TTMI_API int ttmi_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* Asynchronous device-side error flag (out-of-range embedding id): returns TTMI_EINDEX
+ * once after a kernel has raised it.  The caller must have synchronised the stream.
+ * Stands in for the `trap` in gpu_embedding_kernel.cu:32-34 and the throw in
+ * embedding.cpp:59. */
+TTMI_API int ttmi_check_async(void);
+
+/* ---------------------------------------------------- memory-bound epilogue kernels --- */
+
+/* kernels::LayerNorm  (layers/kernels/layer_norm.cpp:33-91, CPU branch :43-74).
+ * In place on out[m,n]: mean = sum/n, var = sumsq/n - mean^2, out = beta + gamma*(x-mean)/sqrt(var+eps). */
+TTMI_API int ttmi_layer_norm(void* out, const void* gamma, const void* beta, int64_t m, int64_t n,
+                             float eps, int dtype, void* stream);
+
+/* kernels::AddBiasLayerNorm  (layers/kernels/layer_norm.cpp:99-180, CPU branch :130-164).
+ * out = LN(out + input + bias), in place on out. */
+TTMI_API int ttmi_add_bias_layer_norm(void* out, const void* input, const void* bias, const void* gamma,
+                                      const void* beta, int64_t m, int64_t n, float eps, int dtype,
+                                      void* stream);
+
+/* kernels::AddBiasAct<T, Act>  (layers/kernels/activation.cpp:33-55, 90-119).
+ * out[m,n] = act(out[m,n] + bias[n]) in place; gelu is the tanh form. */
+TTMI_API int ttmi_add_bias_act(void* out, const void* bias, int64_t m, int64_t n, int act, int dtype,
+                               void* stream);
+
+/* kernels::ApplyMaskAndSoftmax  (layers/kernels/softmax.cpp:28-125).
+ * In place on score[B,h,F,T]: x = score*scale + mask; p = exp(x-max)/sum over T.
+ * `mask` is fp32 or NULL; mask_is_2d != 0 -> mask[B,T] (broadcast over heads and rows),
+ * else mask[B,F,T]. */
+TTMI_API int ttmi_apply_mask_and_softmax(void* score, const float* mask, int64_t batch, int64_t heads,
+                                         int64_t from_len, int64_t to_len, int mask_is_2d, float scale,
+                                         int dtype, void* stream);
+
+/* kernels::SplitAddBiasTransposeForScore, 3-output form  (layers/kernels/transpose.cpp:310-406).
+ * in[B,S,3,h,d] + bias[3,h,d] -> q,k,v each [B,h,S,d]. */
+TTMI_API int ttmi_split_add_bias_transpose_for_score(const void* in, const void* bias, void* q, void* k,
+                                                     void* v, int64_t batch, int64_t seq, int64_t heads,
+                                                     int64_t head_dim, int dtype, void* stream);
+
+/* kernels::SplitAddBiasTransposeForScorePad  (layers/kernels/transpose.cpp:459-580).
+ * Packed in[1,sum(len),3,h,d] -> q,k,v [B,h,max_seq,d]; rows s >= len[b] are zero (no bias).
+ * `cu_seqlens` is a DEVICE int32 array [batch+1] of exclusive prefix sums of the lengths
+ * (built once per batch by ttmi_build_cu_seqlens instead of a per-call malloc+copy,
+ * gpu_transpose_kernel.cu:213-222). */
+TTMI_API int ttmi_split_add_bias_transpose_for_score_pad(const void* in, const void* bias, void* q, void* k,
+                                                         void* v, const int32_t* cu_seqlens, int64_t batch,
+                                                         int64_t max_seq, int64_t heads, int64_t head_dim,
+                                                         int dtype, void* stream);
+
+/* kernels::TransposeForScore  (layers/kernels/transpose.cpp:105-125, 158-191): [B,h,S,d] -> [B,S,h,d]. */
+TTMI_API int ttmi_transpose_for_score(const void* in, void* out, int64_t batch, int64_t seq, int64_t heads,
+                                      int64_t head_dim, int dtype, void* stream);
+
+/* kernels::TransposeForScorePad  (layers/kernels/transpose.cpp:128-156, 589-623):
+ * [B,h,max_seq,d] -> packed [1,sum(len),h,d], pad rows dropped. */
+TTMI_API int ttmi_transpose_for_score_pad(const void* in, void* out, const int32_t* cu_seqlens, int64_t batch,
+                                          int64_t max_seq, int64_t heads, int64_t head_dim, int dtype,
+                                          void* stream);
+
+/* Upload host lengths as a device prefix array cu_seqlens[batch+1] (int32) on `stream`.
+ * `staging` is pinned host memory of at least (batch+1)*4 bytes owned by the caller. */
+TTMI_API int ttmi_build_cu_seqlens(const int64_t* host_lens, int64_t batch, int32_t* staging,
+                                   int32_t* cu_seqlens_dev, void* stream);
+
+/* Per-token destination rows of a packed batch: token_rows[t] = b*max_seq + (t - cu_seqlens[b])
+ * for cu_seqlens[b] <= t < cu_seqlens[b+1]; `total` = cu_seqlens[batch].  Built once per batch;
+ * consumed by the QKV_SPLIT_PAD GEMM epilogue. */
+TTMI_API int ttmi_build_token_rows(const int32_t* cu_seqlens, int64_t batch, int64_t max_seq, int64_t total,
+                                   int32_t* token_rows, void* stream);
+
+/* kernels::LookupEmbedding<Add>  (layers/kernels/embedding.cpp:28-85).
+ * out[i,:] = table[ids[i],:]  (add=0) or out[i,:] += table[ids[i],:] (add=1); ids are int64.
+ * An id outside [0,vocab) leaves the row untouched and raises the async error flag. */
+TTMI_API int ttmi_lookup_embedding(void* out, const void* table, const int64_t* ids, int64_t num_ids,
+                                   int64_t hidden, int64_t vocab, int add, int dtype, void* stream);
+
+/* layers::BERTEmbedding::operator() as one kernel  (layers/bert_embedding.cpp:24-65):
+ * out = LN(word[ids] + type[type_ids] + pos[pos_ids]), adds in that order. */
+TTMI_API int ttmi_bert_embedding(void* out, const int64_t* ids, const int64_t* pos_ids,
+                                 const int64_t* type_ids, const void* word_table, const void* pos_table,
+                                 const void* type_table, const void* gamma, const void* beta,
+                                 int64_t num_ids, int64_t hidden, int64_t vocab, int64_t max_pos,
+                                 int64_t num_types, float eps, int dtype, void* stream);
+
+/* kernels::common::Sequence / Fill / Transform  (layers/kernels/common.cpp:29-90), the three
+ * helpers of layers::PrepareBertMasks (layers/prepare_bert_masks.cpp:24-66). */
+TTMI_API int ttmi_fill_i64(int64_t* data, int64_t n, int64_t value, void* stream);
+TTMI_API int ttmi_fill_f32(float* data, int64_t n, float value, void* stream);
+/* data[r, c] = c for r < rows, c < cols */
+TTMI_API int ttmi_sequence_rows_i64(int64_t* data, int64_t rows, int64_t cols, void* stream);
+/* dst[i] = -10000 * (1 - src[i]) */
+TTMI_API int ttmi_mask_transform(const int64_t* src, float* dst, int64_t n, void* stream);
+
+/* Smart-batch key-padding mask (python layers/modeling_smart_pad.py:465-475):
+ * mask[b, 0, t] = 0 for t < len[b] else -1e9, shape [B,1,max_seq] fp32. */
+TTMI_API int ttmi_smart_pad_mask(float* mask, const int32_t* cu_seqlens, int64_t batch, int64_t max_seq,
+                                 void* stream);
+
+/* Plain 2-D transpose out[c,r] = in[r,c], used once per weight at layer construction to
+ * keep every weight K-contiguous ([out,in]) for the MFMA kernels. */
+TTMI_API int ttmi_transpose_2d(const void* in, void* out, int64_t rows, int64_t cols, int dtype, void* stream);
+
+/* Element type conversion between TTMI_F32 / F16 / BF16 buffers. */
+TTMI_API int ttmi_convert(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, void* stream);
+
+/* ------------------------------------------------------------------ MFMA GEMMs -------- */
+
+/* kernels::MatMul  (layers/kernels/mat_mul.cpp:30-118).
+ * C[M,N] = alpha * A[M,K] * op(B) + beta * C, all row-major with leading dimensions in
+ * elements.  trans_b = 0: B is [K,N] (ldb >= N);  trans_b != 0: B is [N,K] (ldb >= K). */
+TTMI_API int ttmi_gemm(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int64_t lda,
+                       int64_t ldb, int64_t ldc, int trans_b, float alpha, float beta, int dtype,
+                       void* stream);
+
+/* kernels::BatchMatMul  (layers/kernels/mat_mul.cpp:119-213): strided-batched form of the
+ * above; batch_count problems, strides in elements. */
+TTMI_API int ttmi_gemm_strided_batched(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
+                                       int64_t lda, int64_t ldb, int64_t ldc, int64_t stride_a,
+                                       int64_t stride_b, int64_t stride_c, int64_t batch_count, int trans_b,
+                                       float alpha, float beta, int dtype, void* stream);
+
+/* BatchMatMul over a [batch, heads] grid of problems whose operands are strided views:
+ * problem (b, h) uses A + b*a_batch + h*a_head, etc. (strides in elements).  With
+ * c_batch = S*heads*d, c_head = d, ldc = heads*d the P*V product lands directly in
+ * [B,S,h,d], i.e. BatchMatMul + TransposeForScore in one pass
+ * (layers/multi_headed_attention.cpp:345-354). */
+TTMI_API int ttmi_gemm_batched_heads(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
+                                     int64_t lda, int64_t ldb, int64_t ldc, int64_t heads, int64_t a_batch,
+                                     int64_t a_head, int64_t b_batch, int64_t b_head, int64_t c_batch,
+                                     int64_t c_head, int64_t batch, int trans_b, float alpha, float beta,
+                                     int dtype, void* stream);
+
+/* Arguments of the fused epilogues; unused members are NULL / 0. */
+typedef struct ttmi_epilogue_args {
+  const void* bias;          /* [N], same dtype as C                                        */
+  const void* residual;      /* [M,N] row-major, ld = ldc          (BIAS_RESIDUAL)          */
+  int act;                   /* ttmi_act                            (BIAS_ACT)               */
+  void* q; void* k; void* v; /* outputs [B,h,S,d]                   (QKV_SPLIT[_PAD])        */
+  int64_t seq;               /* S (or max_seq for the padded form)                          */
+  int64_t heads;             /* h                                                           */
+  int64_t head_dim;          /* d; N must equal 3*h*d                                       */
+  const int32_t* token_rows; /* device [M]: packed token -> b*max_seq+s (QKV_SPLIT_PAD)      */
+  int64_t batch;             /* B                                   (QKV_SPLIT_PAD)          */
+} ttmi_epilogue_args;
+
+/* MatMul with the following memory-bound op folded into the store of the accumulators:
+ *   BIAS_ACT       = MatMul + AddBiasAct            (layers/bert_intermediate.cpp:43-46)
+ *   BIAS_RESIDUAL  = MatMul + the `out+input+bias` part of AddBiasLayerNorm
+ *                    (layers/bert_output.cpp:47-51, layers/multi_headed_attention.cpp:359-371)
+ *   QKV_SPLIT[_PAD]= MatMul + SplitAddBiasTransposeForScore[Pad]
+ *                    (layers/multi_headed_attention.cpp:199-203, ..._smart_batch.cpp:212-217)
+ * B is always [N,K] here (weights are repacked K-contiguous at construction).
+ * For the QKV forms `c` may be NULL. */
+TTMI_API int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
+                             int64_t lda, int64_t ldb, int64_t ldc, int epilogue,
+                             const ttmi_epilogue_args* args, int dtype, void* stream);
+
+/* int8 path (quantized BERT: int8 x int8 -> int32 accumulators, exact).
+ * ttmi_quantize_rows_i8: per-tensor symmetric dynamic scale from max|x| over the whole
+ *   [m,k] activation: scale = max|x|/127 (1 if the tensor is all zero), q = clamp(rint(x/scale), -127, 127).
+ *   `scale_dev` is a DEVICE float[2]: [0] receives the scale, [1] is scratch for the max.
+ * ttmi_gemm_i8: C_i32[M,N] = A_i8[M,K] * B_i8[N,K]^T.
+ * ttmi_dequant_bias: out[m,n] = acc[m,n] * (*act_scale) * w_scale[n] + bias[n] (fp32 out; bias may be NULL). */
+TTMI_API int ttmi_quantize_rows_i8(const float* x, int8_t* q, float* scale_dev, int64_t m, int64_t k,
+                                   void* stream);
+TTMI_API int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_t n, int64_t k,
+                          int64_t lda, int64_t ldb, int64_t ldc, void* stream);
+TTMI_API int ttmi_dequant_bias(const int32_t* acc, const float* act_scale_dev, const float* w_scale,
+                               const float* bias, float* out, int64_t m, int64_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTMI_H_ */

@@ -1,0 +1,231 @@
+"""GPU parity of the MFMA GEMM family (MatMul, BatchMatMul, fused epilogues, int8) against the
+CPU oracle, through the C ABI.
+
+Inputs are scaled so outputs are O(1); fp32 must agree to 1e-4 (accumulation order only),
+fp16 to 4e-3 and bf16 to 3e-2 max-abs (one storage rounding of an O(1..4) value); int8
+accumulators are compared bit-exactly against an integer brute force.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import ALL_DTYPES, TTMI_DTYPES, dev, host, max_abs, ok, ptr, rounded, stream
+from turbotransformers_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+GEMM_TOL = {"f32": 1e-4, "f16": 4e-3, "bf16": 3e-2}
+
+
+def _ab(rng, M, N, K, b_trans):
+    A = rng.standard_normal((M, K), np.float32)
+    B = (rng.standard_normal((N, K) if b_trans else (K, N), np.float32) / np.sqrt(K)).astype(np.float32)
+    return A, B
+
+
+def test_matmul_known_answer(ttmi):
+    # layers/kernels/mat_mul_test.cpp:29-40: [1,2;3,4] x [2,3;4,5] = [10,13;22,29]
+    A, B = np.array([[1, 2], [3, 4]], np.float32), np.array([[2, 3], [4, 5]], np.float32)
+    for dt in ALL_DTYPES:
+        C = torch.zeros((2, 2), dtype=dev(A, dt).dtype, device="cuda")
+        ok(ttmi.ttmi_gemm(ptr(dev(A, dt)), ptr(dev(B, dt)), ptr(C), 2, 2, 2, 2, 2, 2, 0, 1.0, 0.0, TTMI_DTYPES[dt], stream()))
+        assert np.array_equal(host(C), np.array([[10, 13], [22, 29]], np.float32))
+        ok(ttmi.ttmi_gemm(ptr(dev(A, dt)), ptr(dev(np.ascontiguousarray(B.T), dt)), ptr(C), 2, 2, 2, 2, 2, 2, 1, 1.0, 0.0,
+                          TTMI_DTYPES[dt], stream()))
+        assert np.array_equal(host(C), np.array([[10, 13], [22, 29]], np.float32))
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("b_trans", [0, 1])
+@pytest.mark.parametrize("M,N,K", [
+    (5, 768, 768), (20, 3072, 768), (20, 768, 3072), (128, 2304, 768), (300, 256, 64), (257, 129, 72),
+    (33, 65, 50), (1, 8, 8), (2048, 2304, 768), (8192, 2304, 768), (4100, 1024, 1024), (500, 500, 500)])
+def test_matmul(ttmi, oracle, dt, b_trans, M, N, K):
+    rng = np.random.default_rng(M + N + K + b_trans)
+    A, B = _ab(rng, M, N, K, b_trans)
+    dA, dB = dev(A, dt), dev(B, dt)
+    C = torch.full((M, N), 3.0, dtype=dA.dtype, device="cuda")
+    ok(ttmi.ttmi_gemm(ptr(dA), ptr(dB), ptr(C), M, N, K, K, K if b_trans else N, N, b_trans, 1.0, 0.0,
+                      TTMI_DTYPES[dt], stream()))
+    want = oracle.matmul(rounded(A, dt), rounded(B, dt), bool(b_trans))
+    assert max_abs(host(C), want) <= GEMM_TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+def test_matmul_alpha_beta_and_ld(ttmi, oracle, dt):
+    rng = np.random.default_rng(5)
+    M, N, K, lda, ldb, ldc = 70, 90, 64, 80, 72, 96
+    A = rng.standard_normal((M, lda), np.float32)
+    B = (rng.standard_normal((N, ldb), np.float32) / 8).astype(np.float32)
+    C0 = rng.standard_normal((M, ldc), np.float32)
+    dC = dev(C0, dt)
+    ok(ttmi.ttmi_gemm(ptr(dev(A, dt)), ptr(dev(B, dt)), ptr(dC), M, N, K, lda, ldb, ldc, 1, 0.5, 2.0, TTMI_DTYPES[dt],
+                      stream()))
+    want = rounded(C0, dt).copy()
+    want[:, :N] = 0.5 * (rounded(A, dt)[:, :K].astype(np.float64) @ rounded(B, dt)[:, :K].T.astype(np.float64)) + 2.0 * want[:, :N]
+    got = host(dC)
+    assert max_abs(got[:, :N], want[:, :N]) <= GEMM_TOL[dt] * 3
+    assert np.array_equal(got[:, N:], rounded(C0, dt)[:, N:])  # columns beyond N untouched
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("batch,S,d", [(24, 100, 64), (6, 500, 64), (4, 128, 64), (3, 37, 20)])
+def test_batch_matmul_attention_shapes(ttmi, oracle, dt, batch, S, d):
+    """batch_gemm3 (Q K^T, alpha = 1/sqrt(d)) and batch_gemm4 (P V) of
+    layers/multi_headed_attention.cpp:328-346."""
+    rng = np.random.default_rng(S)
+    Q, Kt, V = (rng.standard_normal((batch, S, d), np.float32) for _ in range(3))
+    alpha = 1.0 / np.sqrt(d)
+    dQ, dK, dV = dev(Q, dt), dev(Kt, dt), dev(V, dt)
+    score = torch.empty((batch, S, S), dtype=dQ.dtype, device="cuda")
+    ok(ttmi.ttmi_gemm_strided_batched(ptr(dQ), ptr(dK), ptr(score), S, S, d, d, d, S, S * d, S * d, S * S, batch, 1,
+                                      alpha, 0.0, TTMI_DTYPES[dt], stream()))
+    want = oracle.batch_matmul(rounded(Q, dt), rounded(Kt, dt), True, alpha)
+    assert max_abs(host(score), want) <= GEMM_TOL[dt] * 4
+    P = (rng.random((batch, S, S), np.float32) / S * 2).astype(np.float32)
+    dP = dev(P, dt)
+    ctx = torch.empty((batch, S, d), dtype=dQ.dtype, device="cuda")
+    ok(ttmi.ttmi_gemm_strided_batched(ptr(dP), ptr(dV), ptr(ctx), S, d, S, S, d, d, S * S, S * d, S * d, batch, 0, 1.0,
+                                      0.0, TTMI_DTYPES[dt], stream()))
+    want = oracle.batch_matmul(rounded(P, dt), rounded(V, dt), False)
+    assert max_abs(host(ctx), want) <= GEMM_TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+def test_batched_heads_writes_merged_layout(ttmi, oracle, dt):
+    """P V with the [B,h,S,d] -> [B,S,h,d] transpose folded into the store."""
+    rng = np.random.default_rng(9)
+    B, h, S, d = 2, 3, 50, 64
+    P = (rng.random((B, h, S, S), np.float32) / S * 2).astype(np.float32)
+    V = rng.standard_normal((B, h, S, d), np.float32)
+    dP, dV = dev(P, dt), dev(V, dt)
+    out = torch.empty((B, S, h, d), dtype=dP.dtype, device="cuda")
+    ok(ttmi.ttmi_gemm_batched_heads(ptr(dP), ptr(dV), ptr(out), S, d, S, S, d, h * d, h, h * S * S, S * S, h * S * d,
+                                    S * d, S * h * d, d, B, 0, 1.0, 0.0, TTMI_DTYPES[dt], stream()))
+    want = oracle.transpose_for_score(oracle.batch_matmul(rounded(P, dt), rounded(V, dt), False))
+    assert max_abs(host(out), want) <= GEMM_TOL[dt]
+
+
+def _epi(**kw):
+    a = capi.EpilogueArgs()
+    for k, v in kw.items():
+        setattr(a, k, v.data_ptr() if isinstance(v, torch.Tensor) else v)
+    return a
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("M,N,K", [(100, 3072, 768), (4096, 3072, 768), (77, 768, 3072)])
+def test_fused_bias_gelu(ttmi, oracle, dt, M, N, K):
+    import ctypes
+    rng = np.random.default_rng(M)
+    A, W = _ab(rng, M, N, K, 1)
+    bias = rng.standard_normal(N).astype(np.float32)
+    dA, dW, db = dev(A, dt), dev(W, dt), dev(bias, dt)
+    C = torch.empty((M, N), dtype=dA.dtype, device="cuda")
+    args = _epi(bias=db, act=capi.ACT_GELU)
+    ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, capi.EPI_BIAS_ACT, ctypes.byref(args),
+                            TTMI_DTYPES[dt], stream()))
+    want = oracle.add_bias_act(oracle.matmul(rounded(A, dt), rounded(W, dt), True), rounded(bias, dt), 0)
+    assert max_abs(host(C), want) <= GEMM_TOL[dt] * 2
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+def test_fused_bias_and_bias_residual(ttmi, oracle, dt):
+    import ctypes
+    rng = np.random.default_rng(11)
+    M, N, K = 300, 768, 768
+    A, W = _ab(rng, M, N, K, 1)
+    bias = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((M, N), np.float32)
+    dA, dW, db, dres = dev(A, dt), dev(W, dt), dev(bias, dt), dev(res, dt)
+    C = torch.empty((M, N), dtype=dA.dtype, device="cuda")
+    base = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    args = _epi(bias=db)
+    ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, capi.EPI_BIAS, ctypes.byref(args),
+                            TTMI_DTYPES[dt], stream()))
+    assert max_abs(host(C), base + rounded(bias, dt)) <= GEMM_TOL[dt] * 2
+    args = _epi(bias=db, residual=dres)
+    ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, capi.EPI_BIAS_RESIDUAL, ctypes.byref(args),
+                            TTMI_DTYPES[dt], stream()))
+    assert max_abs(host(C), base + rounded(bias, dt) + rounded(res, dt)) <= GEMM_TOL[dt] * 3
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 7, 2, 32)])
+def test_fused_qkv_split(ttmi, oracle, dt, B, S, h, d):
+    import ctypes
+    rng = np.random.default_rng(S)
+    H = h * d
+    A, W = _ab(rng, B * S, 3 * H, H, 1)
+    bias = rng.standard_normal(3 * H).astype(np.float32)
+    dA, dW, db = dev(A, dt), dev(W, dt), dev(bias, dt)
+    q, k, v = (torch.empty((B, h, S, d), dtype=dA.dtype, device="cuda") for _ in range(3))
+    args = _epi(bias=db, q=q, k=k, v=v, seq=S, heads=h, head_dim=d)
+    ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), None, B * S, 3 * H, H, H, H, 3 * H, capi.EPI_QKV_SPLIT,
+                            ctypes.byref(args), TTMI_DTYPES[dt], stream()))
+    qkv = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    want = oracle.split_add_bias_transpose(qkv, rounded(bias, dt), B, S, h, d)
+    for got, w in zip((q, k, v), want):
+        assert max_abs(host(got), w) <= GEMM_TOL[dt] * 2
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+def test_fused_qkv_split_pad(ttmi, oracle, dt):
+    import ctypes
+    rng = np.random.default_rng(21)
+    lens = np.array([9, 30, 1, 17], np.int64)
+    h, d = 4, 64
+    H, B, maxS, total = h * d, len(lens), int(lens.max()), int(lens.sum())
+    A, W = _ab(rng, total, 3 * H, H, 1)
+    bias = rng.standard_normal(3 * H).astype(np.float32)
+    dA, dW, db = dev(A, dt), dev(W, dt), dev(bias, dt)
+    cu = np.zeros(B + 1, np.int32)
+    cu[1:] = np.cumsum(lens)
+    rows = torch.empty(total, dtype=torch.int32, device="cuda")
+    ok(ttmi.ttmi_build_token_rows(ptr(dev(cu)), B, maxS, total, ptr(rows), stream()))
+    q, k, v = (torch.zeros((B, h, maxS, d), dtype=dA.dtype, device="cuda") for _ in range(3))
+    args = _epi(bias=db, q=q, k=k, v=v, seq=maxS, heads=h, head_dim=d, token_rows=rows, batch=B)
+    ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), None, total, 3 * H, H, H, H, 3 * H, capi.EPI_QKV_SPLIT_PAD,
+                            ctypes.byref(args), TTMI_DTYPES[dt], stream()))
+    qkv = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    want = oracle.split_add_bias_transpose_pad(qkv, rounded(bias, dt), lens, h, d)
+    for got, w in zip((q, k, v), want):
+        assert max_abs(host(got), w) <= GEMM_TOL[dt] * 2
+
+
+@pytest.mark.parametrize("M,N,K", [(20, 768, 768), (2560, 3072, 768), (2560, 768, 3072), (33, 48, 80), (300, 1000, 130)])
+def test_gemm_i8_accumulators_bit_exact(ttmi, oracle, M, N, K):
+    rng = np.random.default_rng(K)
+    A = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    B = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    C = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    ok(ttmi.ttmi_gemm_i8(ptr(dev(A)), ptr(dev(B)), ptr(C), M, N, K, K, K, N, stream()))
+    want = A.astype(np.int32) @ B.astype(np.int32).T  # exact integer arithmetic
+    assert np.array_equal(host(C), want)
+    if M * N * K < 5e7:
+        assert np.array_equal(want, oracle.gemm_i8(A, B))
+
+
+def test_int8_linear_pipeline(ttmi, oracle):
+    """quantize -> int8 GEMM -> dequant+bias, against the oracle's statement of the same scheme."""
+    rng = np.random.default_rng(3)
+    M, N, K = 200, 384, 256
+    x = rng.standard_normal((M, K), np.float32)
+    w = (rng.standard_normal((N, K), np.float32) * 0.02).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    qw, sw = oracle.quantize_weight_i8(w)
+    qx_want, sx_want = oracle.quantize_tensor_i8(x)
+    dq = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    scale = torch.empty(2, device="cuda")
+    ok(ttmi.ttmi_quantize_rows_i8(ptr(dev(x)), ptr(dq), ptr(scale), M, K, stream()))
+    assert np.array_equal(host(dq), qx_want)
+    assert host(scale)[0] == np.float32(sx_want)
+    acc = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    ok(ttmi.ttmi_gemm_i8(ptr(dq), ptr(dev(qw)), ptr(acc), M, N, K, K, K, N, stream()))
+    acc_want = oracle.gemm_i8(qx_want, qw)
+    assert np.array_equal(host(acc), acc_want)
+    out = torch.empty((M, N), device="cuda")
+    ok(ttmi.ttmi_dequant_bias(ptr(acc), ptr(scale), ptr(dev(sw)), ptr(dev(bias)), ptr(out), M, N, stream()))
+    want = oracle.dequant_bias(acc_want, sx_want, sw, bias)
+    assert max_abs(host(out), want) <= 1e-5
+    assert max_abs(want, x @ w.T + bias) < 0.05  # and the scheme itself approximates the fp32 Linear

@@ -1,0 +1,258 @@
+"""GPU parity of every memory-bound kernel of the C ABI against the CPU oracle.
+
+Shapes follow the reference's own kernel tests (layers/kernels/*_test.cpp): softmax
+B in {1,20}, from/to in 10..500 with 2-D and 3-D masks; LayerNorm H in {768, 2000};
+activations H in {500, 768, 8193}; embeddings H in {128, 768}; transposes with ragged
+lengths.  fp32 is compared at 2e-5, fp16 at 4e-3, bf16 at 2e-2 (max-abs, O(1) outputs);
+pure permutations and gathers are compared bit-exactly.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import ALL_DTYPES, TOL, TTMI_DTYPES, dev, host, max_abs, ok, ptr, rounded, stream
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("m,n", [(7, 768), (130, 1024), (33, 2000), (5, 770), (3, 12288), (64, 128), (1, 8)])
+def test_add_bias_layer_norm(ttmi, oracle, dt, m, n):
+    rng = np.random.default_rng(m * 1000 + n)
+    out, inp = rng.standard_normal((m, n), np.float32), rng.standard_normal((m, n), np.float32)
+    bias, gamma, beta = (rng.standard_normal(n).astype(np.float32) for _ in range(3))
+    d_out = dev(out, dt)
+    ok(ttmi.ttmi_add_bias_layer_norm(ptr(d_out), ptr(dev(inp, dt)), ptr(dev(bias, dt)), ptr(dev(gamma, dt)),
+                                     ptr(dev(beta, dt)), m, n, 1e-12, TTMI_DTYPES[dt], stream()))
+    want = oracle.add_bias_layer_norm(rounded(out, dt), rounded(inp, dt), rounded(bias, dt), rounded(gamma, dt),
+                                      rounded(beta, dt))
+    assert max_abs(host(d_out), want) <= TOL[dt] * 4
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("m,n", [(20, 768), (9, 2000), (4, 100)])
+def test_layer_norm(ttmi, oracle, dt, m, n):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal((m, n), np.float32) * 3 + 1
+    gamma, beta = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    d = dev(x, dt)
+    ok(ttmi.ttmi_layer_norm(ptr(d), ptr(dev(gamma, dt)), ptr(dev(beta, dt)), m, n, 1e-12, TTMI_DTYPES[dt], stream()))
+    want = oracle.layer_norm(rounded(x, dt), rounded(gamma, dt), rounded(beta, dt))
+    assert max_abs(host(d), want) <= TOL[dt] * 4
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("act", [0, 1, 2])
+@pytest.mark.parametrize("m,n", [(20, 500), (20, 768), (3, 8193), (128, 3072)])
+def test_add_bias_act(ttmi, oracle, dt, act, m, n):
+    rng = np.random.default_rng(n + act)
+    x = rng.standard_normal((m, n), np.float32) * 2
+    bias = rng.standard_normal(n).astype(np.float32)
+    d = dev(x, dt)
+    ok(ttmi.ttmi_add_bias_act(ptr(d), ptr(dev(bias, dt)), m, n, act, TTMI_DTYPES[dt], stream()))
+    want = oracle.add_bias_act(rounded(x, dt), rounded(bias, dt), act)
+    assert max_abs(host(d), want) <= TOL[dt] * 4
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("mask_kind", ["2d", "3d", "none"])
+@pytest.mark.parametrize("B,h,F,T", [(1, 12, 10, 10), (20, 12, 40, 100), (2, 3, 128, 128), (2, 2, 500, 500),
+                                     (1, 2, 64, 512), (1, 1, 7, 1030), (1, 1, 3, 2500), (3, 2, 17, 33)])
+def test_apply_mask_and_softmax(ttmi, oracle, dt, mask_kind, B, h, F, T):
+    rng = np.random.default_rng(B * 7 + T)
+    qk = rng.standard_normal((B, h, F, T), np.float32) * 3
+    mask = None
+    if mask_kind == "2d":
+        mask = np.where(rng.random((B, 1, 1, T)) < 0.2, -10000.0, 0.0).astype(np.float32)
+        mask[..., 0] = 0
+    elif mask_kind == "3d":
+        mask = np.where(rng.random((B, 1, F, T)) < 0.2, -10000.0, 0.0).astype(np.float32)
+        mask[..., 0] = 0
+    d = dev(qk, dt)
+    dm = dev(mask) if mask is not None else None
+    ok(ttmi.ttmi_apply_mask_and_softmax(ptr(d), ptr(dm), B, h, F, T, 1 if mask_kind == "2d" else 0, 0.125,
+                                        TTMI_DTYPES[dt], stream()))
+    want = oracle.apply_mask_and_softmax(rounded(qk, dt), mask, 0.125, mask_kind == "2d")
+    got = host(d)
+    assert max_abs(got, want) <= TOL[dt]
+    assert np.allclose(got.sum(-1), 1.0, atol=TOL[dt] * 8 + T * 2e-7 * (0 if dt == "f32" else 30))
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("B,S,h,d", [(1, 10, 12, 64), (3, 17, 4, 64), (2, 5, 3, 20), (2, 128, 16, 64)])
+def test_split_add_bias_transpose(ttmi, oracle, dt, B, S, h, d):
+    rng = np.random.default_rng(S)
+    x = rng.standard_normal((B, S, 3, h, d), np.float32)
+    bias = rng.standard_normal((3, h, d), np.float32)
+    q, k, v = (torch.empty((B, h, S, d), dtype=dev(x, dt).dtype, device="cuda") for _ in range(3))
+    ok(ttmi.ttmi_split_add_bias_transpose_for_score(ptr(dev(x, dt)), ptr(dev(bias, dt)), ptr(q), ptr(k), ptr(v), B, S,
+                                                    h, d, TTMI_DTYPES[dt], stream()))
+    wq, wk, wv = oracle.split_add_bias_transpose(rounded(x, dt), rounded(bias, dt), B, S, h, d)
+    for got, want in ((q, wq), (k, wk), (v, wv)):
+        if dt == "f32":
+            assert np.array_equal(host(got), want)  # one fp32 add per element: bit-exact
+        else:
+            assert max_abs(host(got), want) <= TOL[dt] * 4
+
+
+def _cu(lens):
+    cu = np.zeros(len(lens) + 1, np.int32)
+    cu[1:] = np.cumsum(lens)
+    return cu
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("lens,h,d", [([9, 7, 13], 4, 64), ([4, 1], 12, 64), ([10, 19, 20], 2, 24), ([5], 3, 8)])
+def test_split_add_bias_transpose_pad(ttmi, oracle, dt, lens, h, d):
+    rng = np.random.default_rng(sum(lens))
+    total, B, maxS = sum(lens), len(lens), max(lens)
+    x = rng.standard_normal((total, 3, h, d), np.float32)
+    bias = rng.standard_normal((3, h, d), np.float32)
+    tdt = dev(x, dt).dtype
+    # poison the outputs: pad rows must be written as zeros by the kernel itself
+    q, k, v = (torch.full((B, h, maxS, d), 7.0, dtype=tdt, device="cuda") for _ in range(3))
+    cu = dev(_cu(lens))
+    ok(ttmi.ttmi_split_add_bias_transpose_for_score_pad(ptr(dev(x, dt)), ptr(dev(bias, dt)), ptr(q), ptr(k), ptr(v),
+                                                        ptr(cu), B, maxS, h, d, TTMI_DTYPES[dt], stream()))
+    want = oracle.split_add_bias_transpose_pad(rounded(x, dt), rounded(bias, dt), lens, h, d)
+    for got, w in zip((q, k, v), want):
+        g = host(got)
+        if dt == "f32":
+            assert np.array_equal(g, w)
+        else:
+            assert max_abs(g, w) <= TOL[dt] * 4
+        for b, L in enumerate(lens):  # transpose_test.cpp:242-377: pad rows == 0
+            assert not g[b, :, L:, :].any()
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+def test_transpose_for_score_and_pad(ttmi, oracle, dt):
+    rng = np.random.default_rng(3)
+    B, h, S, d = 3, 4, 21, 64
+    x = rng.standard_normal((B, h, S, d), np.float32)
+    dx = dev(x, dt)
+    out = torch.empty((B, S, h, d), dtype=dx.dtype, device="cuda")
+    ok(ttmi.ttmi_transpose_for_score(ptr(dx), ptr(out), B, S, h, d, TTMI_DTYPES[dt], stream()))
+    assert np.array_equal(host(out), oracle.transpose_for_score(rounded(x, dt)))  # permutation: exact
+    lens = [21, 3, 12]
+    packed = torch.empty((sum(lens), h, d), dtype=dx.dtype, device="cuda")
+    ok(ttmi.ttmi_transpose_for_score_pad(ptr(dx), ptr(packed), ptr(dev(_cu(lens))), B, S, h, d, TTMI_DTYPES[dt],
+                                         stream()))
+    assert np.array_equal(host(packed), oracle.transpose_for_score_pad(rounded(x, dt), lens))
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("hidden", [128, 768, 100])
+def test_lookup_embedding_bit_exact(ttmi, oracle, dt, hidden):
+    rng = np.random.default_rng(hidden)
+    vocab, n = 1000, 257
+    table = rng.standard_normal((vocab, hidden), np.float32)
+    ids = rng.integers(0, vocab, n)
+    ids[0], ids[1] = 0, vocab - 1
+    dtab, dids = dev(table, dt), dev(ids)
+    out = torch.zeros((n, hidden), dtype=dtab.dtype, device="cuda")
+    ok(ttmi.ttmi_lookup_embedding(ptr(out), ptr(dtab), ptr(dids), n, hidden, vocab, 0, TTMI_DTYPES[dt], stream()))
+    want = oracle.lookup_embedding(rounded(table, dt), ids)
+    assert np.array_equal(host(out), want)  # gather: bit-exact in every dtype
+    ok(ttmi.ttmi_lookup_embedding(ptr(out), ptr(dtab), ptr(dids), n, hidden, vocab, 1, TTMI_DTYPES[dt], stream()))
+    got2 = host(out)
+    if dt == "f32":
+        assert np.array_equal(got2, oracle.lookup_embedding(table, ids, out=want.copy(), add=True))
+    else:
+        assert max_abs(got2, 2 * want) <= TOL[dt] * 8
+
+
+def test_lookup_embedding_out_of_range_is_reported(ttmi):
+    table = dev(np.ones((10, 64), np.float32))
+    ids = dev(np.array([1, 10, 2], np.int64))
+    out = torch.zeros((3, 64), device="cuda")
+    ok(ttmi.ttmi_lookup_embedding(ptr(out), ptr(table), ptr(ids), 3, 64, 10, 0, 0, stream()))
+    torch.cuda.synchronize()
+    assert ttmi.ttmi_check_async() == -4  # TTMI_EINDEX, where embedding.cpp:59 throws
+    assert ttmi.ttmi_check_async() == 0   # flag is cleared by the read
+    got = host(out)
+    assert got[0].all() and not got[1].any() and got[2].all()
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("hidden", [768, 128, 1024])
+def test_bert_embedding_fused(ttmi, oracle, dt, hidden):
+    rng = np.random.default_rng(hidden + 1)
+    vocab, max_pos, B, S = 3000, 512, 3, 50
+    word, pos, typ = (rng.standard_normal((r, hidden), np.float32) * 0.02 for r in (vocab, max_pos, 2))
+    gamma, beta = 1 + 0.1 * rng.standard_normal(hidden).astype(np.float32), 0.1 * rng.standard_normal(hidden).astype(np.float32)
+    ids = rng.integers(0, vocab, (B, S))
+    pos_ids = np.tile(np.arange(S), (B, 1))
+    type_ids = rng.integers(0, 2, (B, S))
+    dw = dev(word, dt)
+    out = torch.empty((B, S, hidden), dtype=dw.dtype, device="cuda")
+    ok(ttmi.ttmi_bert_embedding(ptr(out), ptr(dev(ids)), ptr(dev(pos_ids)), ptr(dev(type_ids)), ptr(dw),
+                                ptr(dev(pos, dt)), ptr(dev(typ, dt)), ptr(dev(gamma, dt)), ptr(dev(beta, dt)), B * S,
+                                hidden, vocab, max_pos, 2, 1e-12, TTMI_DTYPES[dt], stream()))
+    want = oracle.bert_embedding(ids, pos_ids, type_ids, rounded(word, dt), rounded(pos, dt), rounded(typ, dt),
+                                 rounded(gamma, dt), rounded(beta, dt))
+    # LN amplifies the storage rounding of the three-table sum (values ~0.03) by 1/std ~ 30
+    assert max_abs(host(out), want) <= {"f32": 5e-5, "f16": 3e-2, "bf16": 2.5e-1}[dt]
+
+
+def test_prepare_bert_masks_helpers(ttmi, oracle):
+    B, S = 3, 17
+    rng = np.random.default_rng(0)
+    mask = (rng.random((B, S)) < 0.7).astype(np.int64)
+    pos = torch.empty((B, S), dtype=torch.int64, device="cuda")
+    ones = torch.empty((B, S), dtype=torch.int64, device="cuda")
+    ext = torch.empty((B, 1, 1, S), device="cuda")
+    ok(ttmi.ttmi_sequence_rows_i64(ptr(pos), B, S, stream()))
+    ok(ttmi.ttmi_fill_i64(ptr(ones), B * S, 1, stream()))
+    ok(ttmi.ttmi_mask_transform(ptr(dev(mask)), ptr(ext), B * S, stream()))
+    _, _, want_pos, want_ext = oracle.prepare_bert_masks(B, S, att_mask=mask)
+    assert np.array_equal(host(pos), want_pos)
+    assert np.array_equal(host(ones), np.ones((B, S), np.int64))
+    assert np.array_equal(host(ext), want_ext)
+    f = torch.empty(100, device="cuda")
+    ok(ttmi.ttmi_fill_f32(ptr(f), 100, 2.5, stream()))
+    assert np.array_equal(host(f), np.full(100, 2.5, np.float32))
+
+
+def test_cu_seqlens_token_rows_and_pad_mask(ttmi):
+    lens = np.array([5, 1, 9, 3], np.int64)
+    B, maxS, total = len(lens), int(lens.max()), int(lens.sum())
+    staging = torch.empty(B + 1, dtype=torch.int32).pin_memory()
+    cu = torch.empty(B + 1, dtype=torch.int32, device="cuda")
+    ok(ttmi.ttmi_build_cu_seqlens(lens.ctypes.data_as(ctypes.c_void_p), B, ctypes.c_void_p(staging.data_ptr()), ptr(cu),
+                                  stream()))
+    assert np.array_equal(host(cu), _cu(lens))
+    rows = torch.empty(total, dtype=torch.int32, device="cuda")
+    ok(ttmi.ttmi_build_token_rows(ptr(cu), B, maxS, total, ptr(rows), stream()))
+    want = np.concatenate([b * maxS + np.arange(L) for b, L in enumerate(lens)])
+    assert np.array_equal(host(rows), want)
+    mask = torch.empty((B, 1, maxS), device="cuda")
+    ok(ttmi.ttmi_smart_pad_mask(ptr(mask), ptr(cu), B, maxS, stream()))
+    want_mask = np.where(np.arange(maxS)[None, :] < lens[:, None], 0.0, -1e9).astype(np.float32)
+    assert np.array_equal(host(mask)[:, 0, :], want_mask)
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+def test_transpose_2d_and_convert(ttmi, dt):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((70, 130), np.float32)
+    dx = dev(x, dt)
+    out = torch.empty((130, 70), dtype=dx.dtype, device="cuda")
+    ok(ttmi.ttmi_transpose_2d(ptr(dx), ptr(out), 70, 130, TTMI_DTYPES[dt], stream()))
+    assert np.array_equal(host(out), rounded(x, dt).T)
+    f = torch.empty((70, 130), device="cuda")
+    ok(ttmi.ttmi_convert(ptr(dx), TTMI_DTYPES[dt], ptr(f), 0, 70 * 130, stream()))
+    assert np.array_equal(host(f), rounded(x, dt))
+
+
+def test_memcpy_and_memset(ttmi):
+    a = np.arange(1000, dtype=np.float32)
+    d = torch.empty(1000, device="cuda")
+    ok(ttmi.ttmi_memcpy(ptr(d), a.ctypes.data_as(ctypes.c_void_p), a.nbytes, 0, stream()))
+    back = np.empty_like(a)
+    ok(ttmi.ttmi_memcpy(back.ctypes.data_as(ctypes.c_void_p), ptr(d), a.nbytes, 1, stream()))
+    assert np.array_equal(a, back)
+    ok(ttmi.ttmi_memset_zero(ptr(d), a.nbytes, stream()))
+    assert not host(d).any()

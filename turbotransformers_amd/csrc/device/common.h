@@ -1,0 +1,116 @@
+// Shared device-side helpers for the gfx950 kernels: element types, 16-byte vector
+// access, wave64 reductions and the error plumbing of the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdio>
+#include <string>
+
+#include "ttmi.h"
+
+namespace ttmi {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+using f16 = _Float16;
+using bf16 = __bf16;
+
+// ---- error plumbing -------------------------------------------------------------------
+void set_error(const std::string& msg);
+int fail(int code, const std::string& msg);
+int check_hip(hipError_t e, const char* what);
+
+#define TTMI_HIP(expr)                                   \
+  do {                                                   \
+    int _rc = ::ttmi::check_hip((expr), #expr);          \
+    if (_rc != 0) return _rc;                            \
+  } while (0)
+
+#define TTMI_REQUIRE(cond, msg)                                            \
+  do {                                                                     \
+    if (!(cond)) return ::ttmi::fail(TTMI_EINVAL, std::string(msg) + " [" #cond "]"); \
+  } while (0)
+
+inline int launch_status(const char* what) { return check_hip(hipGetLastError(), what); }
+
+int* async_error_flag();  // device-visible pinned int, 0 = ok
+
+// ---- scalar conversion ----------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float to_float(T v) { return static_cast<float>(v); }
+template <typename T>
+__device__ __forceinline__ T from_float(float v) { return static_cast<T>(v); }
+
+// ---- 16-byte vectors of N elements -----------------------------------------------------
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Vec {
+  T v[N];
+};
+
+template <typename T, int N>
+__device__ __forceinline__ Vec<T, N> load_vec(const T* p) {
+  return *reinterpret_cast<const Vec<T, N>*>(p);
+}
+template <typename T, int N>
+__device__ __forceinline__ void store_vec(T* p, const Vec<T, N>& x) {
+  *reinterpret_cast<Vec<T, N>*>(p) = x;
+}
+
+// ---- wave64 reductions over groups of G lanes (G power of two <= 64) -------------------
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+template <int G>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// tanh-form GELU exactly as the reference states it, written through the logistic identity
+// 0.5*(1+tanh(u)) == 1/(1+exp(-2u)) so it costs one v_exp_f32 and one v_rcp_f32.
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return x * __frcp_rn(1.0f + __expf(-2.0f * u));
+}
+__device__ __forceinline__ float fast_tanh(float x) {
+  // tanh(x) = 1 - 2/(exp(2x)+1); saturates cleanly at +-1 when exp overflows/underflows
+  return 1.0f - 2.0f * __frcp_rn(__expf(2.0f * x) + 1.0f);
+}
+
+template <int ACT>
+__device__ __forceinline__ float apply_act(float x) {
+  if (ACT == TTMI_ACT_GELU) return gelu_tanh(x);
+  if (ACT == TTMI_ACT_TANH) return fast_tanh(x);
+  return fmaxf(x, 0.0f);
+}
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+inline size_t dtype_size(int dtype) {
+  switch (dtype) {
+    case TTMI_F32: return 4;
+    case TTMI_F16: return 2;
+    case TTMI_BF16: return 2;
+    case TTMI_I8: return 1;
+    case TTMI_I32: return 4;
+    case TTMI_I64: return 8;
+    default: return 0;
+  }
+}
+
+// Dispatch a generic lambda on the floating storage type.
+#define TTMI_DISPATCH_FLOAT(dtype, T, ...)                                  \
+  switch (dtype) {                                                          \
+    case TTMI_F32: { using T = float; __VA_ARGS__; break; }                 \
+    case TTMI_F16: { using T = ::ttmi::f16; __VA_ARGS__; break; }           \
+    case TTMI_BF16: { using T = ::ttmi::bf16; __VA_ARGS__; break; }         \
+    default: return ::ttmi::fail(TTMI_EINVAL, "unsupported dtype");         \
+  }
+
+}  // namespace ttmi

@@ -1,0 +1,540 @@
+// MFMA GEMM family for gfx950 (CDNA4).
+//
+//   C[M,N] (+)= A[M,K] * op(B)        A row-major, K contiguous
+//   op(B) = B[N,K]^T  ("NK": weights kept K-contiguous, the fast path)
+//         | B[K,N]    ("KN": P*V and the generic MatMul)
+//
+// One kernel template serves fp16, bf16, fp32 and int8: operands move through LDS as
+// 16-byte chunks (8 halfs / 4 floats / 16 int8), and one chunk per lane is exactly one
+// MFMA operand:
+//   fp16/bf16  v_mfma_f32_32x32x16_{f16,bf16}   lane l: row l%32, k = 8*(l/32)..+7
+//   int8       v_mfma_i32_32x32x32_i8           lane l: row l%32, k = 16*(l/32)..+15
+//   fp32       4 x v_mfma_f32_32x32x2_f32       lane l: row l%32, k = 4*(l/32)+j, j = MFMA index
+// (the k order inside a chunk is the same permutation for A and B, so the sum is unchanged).
+//
+// A workgroup owns a BM x BN tile of C; its WM x WN wavefronts each own a
+// (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA blocks held in fp32/int32 accumulators.
+// K advances in steps of 128 bytes per row; LDS is double-buffered (global loads for step
+// i+1 are issued into registers before the MFMAs of step i and written to the other stage
+// afterwards, one barrier per step).  LDS rows are 128 bytes = 8 chunks, XOR-swizzled by
+// row so that the 32 rows an MFMA operand read touches spread over all banks.
+//
+// Block ids are remapped so that the workgroups resident on one XCD (ids equal mod 8)
+// cover neighbouring tiles and share A rows / the weight matrix in that XCD's L2.
+#include "common.h"
+
+namespace ttmi {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef int intx16 __attribute__((ext_vector_type(16)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// 16 bytes moved as one unit.  may_alias: chunks are views of T-typed memory (global, LDS and
+// small per-lane staging arrays), so type-based alias analysis must not reorder them.
+struct __attribute__((may_alias)) alignas(16) Chunk {
+  uint32_t w[4];
+};
+
+template <typename T, int N>
+__device__ __forceinline__ Chunk pack_chunk(const T (&tmp)[N]) {
+  static_assert(sizeof(T) * N == 16, "a chunk is 16 bytes");
+  Chunk c;
+  __builtin_memcpy(&c, tmp, 16);
+  return c;
+}
+
+constexpr int kRowBytes = 128;   // bytes of K per LDS row and per K step
+constexpr int kChunks = 8;       // 16-byte chunks per LDS row
+constexpr int kNumXcd = 8;
+
+template <typename T>
+struct Mma;
+
+template <>
+struct Mma<f16> {
+  using Acc = floatx16;
+  using AccScalar = float;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<bf16> {
+  using Acc = floatx16;
+  using AccScalar = float;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<float> {
+  using Acc = floatx16;
+  using AccScalar = float;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      c = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a.w[j]), __builtin_bit_cast(float, b.w[j]), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<int8_t> {
+  using Acc = intx16;
+  using AccScalar = int;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), c, 0, 0, 0);
+  }
+};
+
+// Exact unsigned division by a runtime constant (n < 2^31), for row -> (batch, position).
+struct FastDiv {
+  uint32_t mul = 0, shr = 0, d = 1;
+  FastDiv() = default;
+  explicit FastDiv(uint32_t denom) : d(denom) {
+    if (denom <= 1) { mul = 0; shr = 0; d = 1; return; }
+    uint32_t lg = 0;
+    while ((1ull << lg) < denom) ++lg;
+    const uint32_t p = 31 + lg;
+    mul = (uint32_t)(((1ull << p) + denom - 1) / denom);
+    shr = p - 32;
+  }
+  __device__ __forceinline__ uint32_t div(uint32_t n) const { return d == 1 ? n : (__umulhi(n, mul) >> shr); }
+};
+
+struct GemmArgs {
+  const char* a;
+  const char* b;
+  int m, n, k;
+  int64_t lda, ldb;              // elements
+  // batch z -> (z / inner, z % inner); offsets in elements
+  int inner;
+  int64_t a_outer, a_inner, b_outer, b_inner;
+  int tiles_m, tiles_n;
+};
+
+// ------------------------------------------------------------------------ epilogues -----
+// Each epilogue sees (batch z, row m, column n, accumulator value) once per element; lanes
+// of a wavefront hold 32 consecutive columns of one row, so stores are 64..128-byte runs.
+template <typename T>
+struct EpiAlphaBeta {
+  T* c;
+  int64_t ldc, c_outer, c_inner;
+  int inner;
+  float alpha, beta;
+  __device__ __forceinline__ float col(int) const { return 0.f; }
+  __device__ __forceinline__ void store(int z, int m, int n, float v, float) const {
+    T* p = c + (int64_t)(z / inner) * c_outer + (int64_t)(z % inner) * c_inner + (int64_t)m * ldc + n;
+    float r = alpha * v;
+    if (beta != 0.f) r += beta * to_float(*p);
+    *p = from_float<T>(r);
+  }
+};
+
+template <typename T, int ACT, bool HAS_ACT, bool HAS_RES>
+struct EpiBias {
+  T* c;
+  const T* bias;
+  const T* residual;
+  int64_t ldc;
+  __device__ __forceinline__ float col(int n) const { return to_float(bias[n]); }
+  __device__ __forceinline__ void store(int, int m, int n, float v, float bias_n) const {
+    float r = v + bias_n;
+    if (HAS_ACT) r = apply_act<ACT>(r);
+    if (HAS_RES) r += to_float(residual[(int64_t)m * ldc + n]);
+    c[(int64_t)m * ldc + n] = from_float<T>(r);
+  }
+};
+
+// acc + bias -> q,k,v[B,h,S,d].  Row m is token (b,s); PAD: packed token -> padded row through
+// the per-token map token_rows[m] = b*max_seq + s.
+template <typename T, bool PAD>
+struct EpiQkvSplit {
+  T* q;
+  T* k;
+  T* v;
+  const T* bias;
+  const int32_t* token_rows;
+  int seq, heads, dim, hidden;
+  FastDiv div_seq, div_hidden, div_dim;
+  __device__ __forceinline__ float col(int n) const { return to_float(bias[n]); }
+  __device__ __forceinline__ void store(int, int m, int n, float val, float bias_n) const {
+    uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;  // b*seq + s
+    const uint32_t b = div_seq.div(prow);
+    const uint32_t s = prow - b * seq;
+    const uint32_t w = div_hidden.div((uint32_t)n);
+    const uint32_t rem = n - w * hidden;
+    const uint32_t head = div_dim.div(rem);
+    const uint32_t i = rem - head * dim;
+    T* base = (w == 0) ? q : (w == 1 ? k : v);
+    base[(((int64_t)b * heads + head) * seq + s) * dim + i] = from_float<T>(val + bias_n);
+  }
+};
+
+struct EpiInt32 {
+  int32_t* c;
+  int64_t ldc;
+  __device__ __forceinline__ int col(int) const { return 0; }
+  __device__ __forceinline__ void store(int, int m, int n, int v, int) const { c[(int64_t)m * ldc + n] = v; }
+};
+
+// -------------------------------------------------------------------------- kernel ------
+__device__ __forceinline__ int swizzle(int row, int chunk) { return chunk ^ (row & 7); }
+
+template <typename T, int BM, int BN, int WM, int WN, bool B_KN, bool ALIGNED, typename Epi>
+__global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g, const Epi epi) {
+  constexpr int NT = WM * WN * kWave;
+  constexpr int KPC = 16 / sizeof(T);          // elements per chunk
+  constexpr int BK = kRowBytes / sizeof(T);    // elements of K per step
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_ITERS = BM * kChunks / NT, B_ITERS = BN * kChunks / NT;
+  static_assert(BM * kChunks % NT == 0 && BN * kChunks % NT == 0, "tile/threads mismatch");
+  constexpr int KN_CPR = BN * (int)sizeof(T) / 16;  // chunks per k-row of a KN tile
+  using Acc = typename Mma<T>::Acc;
+  using AccScalar = typename Mma<T>::AccScalar;
+
+  extern __shared__ __align__(16) char smem[];
+
+  // XCD-aware tile order: ids equal mod 8 run on one XCD; give each XCD a contiguous tile range.
+  const int tiles = g.tiles_m * g.tiles_n;
+  const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
+  const int logical = (int)(blockIdx.x % kNumXcd) * per_xcd + (int)(blockIdx.x / kNumXcd);
+  if (logical >= tiles) return;
+  const int tile_m = logical / g.tiles_n, tile_n = logical % g.tiles_n;
+  const int z = blockIdx.z;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const T* A = reinterpret_cast<const T*>(g.a) + (int64_t)(z / g.inner) * g.a_outer + (int64_t)(z % g.inner) * g.a_inner;
+  const T* B = reinterpret_cast<const T*>(g.b) + (int64_t)(z / g.inner) * g.b_outer + (int64_t)(z % g.inner) * g.b_inner;
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave, wave = tid / kWave;
+  const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
+  const int lrow = lane & 31, lhalf = lane >> 5;
+
+  Acc acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  Chunk ra[A_ITERS], rb[B_ITERS];
+
+  auto load_chunk = [&](const T* base, int64_t ld, int row, int row_limit, int kcol, int k_limit) -> Chunk {
+    // 16 bytes of row `row`, elements kcol..kcol+KPC-1; zero outside [0,row_limit) x [0,k_limit)
+    Chunk c{{0u, 0u, 0u, 0u}};
+    if (row < row_limit && kcol < k_limit) {
+      const T* p = base + (int64_t)row * ld + kcol;
+      if (ALIGNED) {
+        c = *reinterpret_cast<const Chunk*>(p);
+      } else {
+        T tmp[KPC];
+#pragma unroll
+        for (int e = 0; e < KPC; ++e) tmp[e] = (kcol + e < k_limit) ? p[e] : T(0);
+        c = pack_chunk(tmp);
+      }
+    }
+    return c;
+  };
+
+  auto load_global = [&](int kt) {
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_ITERS; ++i) {
+      const int c = i * NT + tid;
+      ra[i] = load_chunk(A, g.lda, m0 + (c >> 3), g.m, k0 + (c & 7) * KPC, g.k);
+    }
+#pragma unroll
+    for (int i = 0; i < B_ITERS; ++i) {
+      const int c = i * NT + tid;
+      if (!B_KN) {
+        rb[i] = load_chunk(B, g.ldb, n0 + (c >> 3), g.n, k0 + (c & 7) * KPC, g.k);
+      } else {
+        // B[K,N]: row = k index, columns = n
+        rb[i] = load_chunk(B, g.ldb, k0 + c / KN_CPR, g.k, n0 + (c % KN_CPR) * KPC, g.n);
+      }
+    }
+  };
+
+  auto store_lds = [&](int stage) {
+    char* as = smem + stage * STAGE;
+    char* bs = as + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < A_ITERS; ++i) {
+      const int c = i * NT + tid;
+      const int row = c >> 3;
+      *reinterpret_cast<Chunk*>(as + row * kRowBytes + swizzle(row, c & 7) * 16) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_ITERS; ++i) {
+      const int c = i * NT + tid;
+      if (!B_KN) {
+        const int row = c >> 3;
+        *reinterpret_cast<Chunk*>(bs + row * kRowBytes + swizzle(row, c & 7) * 16) = rb[i];
+      } else {
+        *reinterpret_cast<Chunk*>(bs + c * 16) = rb[i];  // plain [k][n]
+      }
+    }
+  };
+
+  auto compute = [&](int stage) {
+    const char* as = smem + stage * STAGE;
+    const char* bs = as + A_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < kChunks / 2; ++kk) {
+      Chunk fa[TM], fb[TN];
+      const int ch = 2 * kk + lhalf;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row = wm0 + i * 32 + lrow;
+        fa[i] = *reinterpret_cast<const Chunk*>(as + row * kRowBytes + swizzle(row, ch) * 16);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = wn0 + j * 32 + lrow;
+        if (!B_KN) {
+          fb[j] = *reinterpret_cast<const Chunk*>(bs + col * kRowBytes + swizzle(col, ch) * 16);
+        } else {
+          const T* bt = reinterpret_cast<const T*>(bs);
+          T tmp[KPC];
+#pragma unroll
+          for (int e = 0; e < KPC; ++e) tmp[e] = bt[(ch * KPC + e) * BN + col];
+          fb[j] = pack_chunk(tmp);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) Mma<T>::run(fa[i], fb[j], acc[i][j]);
+    }
+  };
+
+  const int ksteps = (g.k + BK - 1) / BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < ksteps; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < ksteps) load_global(kt + 1);
+    compute(cur);
+    if (kt + 1 < ksteps) store_lds(cur ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: acc[i][j][e] is C[row = 8*(e/4) + 4*lhalf + e%4][col = lrow] of its 32x32 block
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn0 + j * 32 + lrow;
+    if (n >= g.n) continue;
+    const auto cstate = epi.col(n);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm0 + i * 32 + 8 * (e / 4) + 4 * lhalf + (e % 4);
+        if (m < g.m) epi.store(z, m, n, (AccScalar)acc[i][j][e], cstate);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------ launching -----
+template <typename T, int BM, int BN, int WM, int WN, bool B_KN, bool ALIGNED, typename Epi>
+static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
+  constexpr int NT = WM * WN * kWave;
+  constexpr int LDS = 2 * (BM + BN) * kRowBytes;
+  g.tiles_m = (g.m + BM - 1) / BM;
+  g.tiles_n = (g.n + BN - 1) / BN;
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  TTMI_REQUIRE(tiles < (1ll << 30) && batch < 65536, "GEMM grid too large");
+  const unsigned grid_x = (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd);
+  auto kern = gemm_kernel<T, BM, BN, WM, WN, B_KN, ALIGNED, Epi>;
+  if (LDS > 64 * 1024) {
+    static bool attr_set = false;  // per instantiation
+    if (!attr_set) {
+      TTMI_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+      attr_set = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3(grid_x, 1, (unsigned)batch), dim3(NT), LDS, s, g, epi);
+  return launch_status("gemm_kernel");
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// Tile choice: the largest tile that still gives every CU work.  256x256 needs >= ~1 wave of
+// workgroups over 256 CUs to pay off; small problems (B=1, S=128) take 64x64 tiles.
+template <typename T, bool B_KN, typename Epi>
+static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipStream_t s) {
+  if (g.m <= 0 || g.n <= 0 || batch <= 0) return 0;
+  TTMI_REQUIRE(g.k > 0, "K must be positive");
+  auto tiles = [&](int bm, int bn) { return (int64_t)ceil_div(g.m, bm) * ceil_div(g.n, bn) * batch; };
+  if (!B_KN) {
+    if (aligned) {
+      if (tiles(256, 256) >= 200 && g.n >= 192 && g.m >= 192) return launch_config<T, 256, 256, 2, 4, false, true, Epi>(g, epi, batch, s);
+      if (tiles(128, 128) >= 200) return launch_config<T, 128, 128, 2, 2, false, true, Epi>(g, epi, batch, s);
+      return launch_config<T, 64, 64, 2, 2, false, true, Epi>(g, epi, batch, s);
+    }
+    return launch_config<T, 64, 64, 2, 2, false, false, Epi>(g, epi, batch, s);
+  } else {
+    if (aligned) {
+      if (tiles(128, 128) >= 200 && g.n >= 96) return launch_config<T, 128, 128, 2, 2, true, true, Epi>(g, epi, batch, s);
+      return launch_config<T, 64, 64, 2, 2, true, true, Epi>(g, epi, batch, s);
+    }
+    return launch_config<T, 64, 64, 2, 2, true, false, Epi>(g, epi, batch, s);
+  }
+}
+
+template <typename T>
+static int gemm_alpha_beta(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int64_t lda,
+                           int64_t ldb, int64_t ldc, int inner, int64_t a_outer, int64_t a_inner,
+                           int64_t b_outer, int64_t b_inner, int64_t c_outer, int64_t c_inner, int64_t batch,
+                           int trans_b, float alpha, float beta, hipStream_t s) {
+  TTMI_REQUIRE(m < (1ll << 31) && n < (1ll << 31) && k < (1ll << 31), "dimension too large");
+  GemmArgs g{};
+  g.a = (const char*)a;
+  g.b = (const char*)b;
+  g.m = (int)m; g.n = (int)n; g.k = (int)k;
+  g.lda = lda; g.ldb = ldb;
+  g.inner = inner;
+  g.a_outer = a_outer; g.a_inner = a_inner; g.b_outer = b_outer; g.b_inner = b_inner;
+  EpiAlphaBeta<T> epi{(T*)c, ldc, c_outer, c_inner, inner, alpha, beta};
+  constexpr int KPC = 16 / sizeof(T);
+  auto mult = [](int64_t v) { return v % KPC == 0; };
+  bool aligned = aligned16(a) && aligned16(b) && mult(lda) && mult(ldb) && mult(a_outer) && mult(a_inner) &&
+                 mult(b_outer) && mult(b_inner);
+  if (trans_b) {
+    aligned = aligned && mult(k);
+    return launch_gemm<T, false>(g, epi, (int)batch, aligned, s);
+  }
+  aligned = aligned && mult(k) && mult(n);
+  return launch_gemm<T, true>(g, epi, (int)batch, aligned, s);
+}
+
+}  // namespace ttmi
+
+using namespace ttmi;
+
+extern "C" {
+
+int ttmi_gemm(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+              int64_t ldc, int trans_b, float alpha, float beta, int dtype, void* stream) {
+  TTMI_REQUIRE(a && b && c, "null matrix");
+  TTMI_REQUIRE(lda >= k && ldc >= n && ldb >= (trans_b ? k : n), "leading dimension too small");
+  TTMI_DISPATCH_FLOAT(dtype, T, return gemm_alpha_beta<T>(a, b, c, m, n, k, lda, ldb, ldc, 1, 0, 0, 0, 0, 0, 0, 1,
+                                                          trans_b, alpha, beta, (hipStream_t)stream));
+  return 0;
+}
+
+int ttmi_gemm_strided_batched(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int64_t lda,
+                              int64_t ldb, int64_t ldc, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                              int64_t batch_count, int trans_b, float alpha, float beta, int dtype, void* stream) {
+  TTMI_REQUIRE(a && b && c, "null matrix");
+  TTMI_REQUIRE(lda >= k && ldc >= n && ldb >= (trans_b ? k : n), "leading dimension too small");
+  TTMI_REQUIRE(batch_count >= 0 && batch_count < 65536, "batch_count out of range");
+  TTMI_DISPATCH_FLOAT(dtype, T, return gemm_alpha_beta<T>(a, b, c, m, n, k, lda, ldb, ldc, 1, stride_a, 0, stride_b,
+                                                          0, stride_c, 0, batch_count, trans_b, alpha, beta,
+                                                          (hipStream_t)stream));
+  return 0;
+}
+
+int ttmi_gemm_batched_heads(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int64_t lda,
+                            int64_t ldb, int64_t ldc, int64_t heads, int64_t a_batch, int64_t a_head,
+                            int64_t b_batch, int64_t b_head, int64_t c_batch, int64_t c_head, int64_t batch,
+                            int trans_b, float alpha, float beta, int dtype, void* stream) {
+  TTMI_REQUIRE(a && b && c, "null matrix");
+  TTMI_REQUIRE(heads > 0 && batch >= 0 && batch * heads < 65536, "batch*heads out of range");
+  TTMI_DISPATCH_FLOAT(dtype, T, return gemm_alpha_beta<T>(a, b, c, m, n, k, lda, ldb, ldc, (int)heads, a_batch,
+                                                          a_head, b_batch, b_head, c_batch, c_head, batch * heads,
+                                                          trans_b, alpha, beta, (hipStream_t)stream));
+  return 0;
+}
+
+int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int64_t lda,
+                    int64_t ldb, int64_t ldc, int epilogue, const ttmi_epilogue_args* args, int dtype,
+                    void* stream) {
+  TTMI_REQUIRE(a && b && args, "null argument");
+  TTMI_REQUIRE(m < (1ll << 31) && n < (1ll << 31) && k < (1ll << 31), "dimension too large");
+  TTMI_REQUIRE(lda >= k && ldb >= k, "leading dimension too small");
+  hipStream_t s = (hipStream_t)stream;
+  GemmArgs g{};
+  g.a = (const char*)a;
+  g.b = (const char*)b;
+  g.m = (int)m; g.n = (int)n; g.k = (int)k;
+  g.lda = lda; g.ldb = ldb;
+  g.inner = 1;
+  TTMI_DISPATCH_FLOAT(dtype, T, {
+    constexpr int KPC = 16 / sizeof(T);
+    const bool aligned = aligned16(a) && aligned16(b) && lda % KPC == 0 && ldb % KPC == 0 && k % KPC == 0;
+    switch (epilogue) {
+      case TTMI_EPI_BIAS: {
+        TTMI_REQUIRE(c && args->bias && ldc >= n, "BIAS epilogue needs c and bias");
+        EpiBias<T, 0, false, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc};
+        return (launch_gemm<T, false>(g, epi, 1, aligned, s));
+      }
+      case TTMI_EPI_BIAS_ACT: {
+        TTMI_REQUIRE(c && args->bias && ldc >= n, "BIAS_ACT epilogue needs c and bias");
+        if (args->act == TTMI_ACT_GELU) {
+          EpiBias<T, TTMI_ACT_GELU, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc};
+          return (launch_gemm<T, false>(g, epi, 1, aligned, s));
+        } else if (args->act == TTMI_ACT_TANH) {
+          EpiBias<T, TTMI_ACT_TANH, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc};
+          return (launch_gemm<T, false>(g, epi, 1, aligned, s));
+        } else if (args->act == TTMI_ACT_RELU) {
+          EpiBias<T, TTMI_ACT_RELU, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc};
+          return (launch_gemm<T, false>(g, epi, 1, aligned, s));
+        }
+        return fail(TTMI_EINVAL, "unknown activation");
+      }
+      case TTMI_EPI_BIAS_RESIDUAL: {
+        TTMI_REQUIRE(c && args->bias && args->residual && ldc >= n, "BIAS_RESIDUAL epilogue needs c, bias, residual");
+        EpiBias<T, 0, false, true> epi{(T*)c, (const T*)args->bias, (const T*)args->residual, ldc};
+        return (launch_gemm<T, false>(g, epi, 1, aligned, s));
+      }
+      case TTMI_EPI_QKV_SPLIT:
+      case TTMI_EPI_QKV_SPLIT_PAD: {
+        const bool pad = epilogue == TTMI_EPI_QKV_SPLIT_PAD;
+        TTMI_REQUIRE(args->q && args->k && args->v && args->bias, "QKV epilogue needs q, k, v, bias");
+        TTMI_REQUIRE(args->seq > 0 && args->heads > 0 && args->head_dim > 0, "QKV epilogue needs seq/heads/head_dim");
+        TTMI_REQUIRE(n == 3 * args->heads * args->head_dim, "N must be 3*heads*head_dim");
+        if (pad) TTMI_REQUIRE(args->token_rows != nullptr && args->batch > 0, "padded QKV epilogue needs token_rows and batch");
+        else TTMI_REQUIRE(m % args->seq == 0, "M must be a multiple of seq");
+        const int hidden = (int)(args->heads * args->head_dim);
+        if (pad) {
+          EpiQkvSplit<T, true> epi{(T*)args->q, (T*)args->k, (T*)args->v, (const T*)args->bias, args->token_rows,
+                                   (int)args->seq, (int)args->heads, (int)args->head_dim, hidden,
+                                   FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim)};
+          return (launch_gemm<T, false>(g, epi, 1, aligned, s));
+        }
+        EpiQkvSplit<T, false> epi{(T*)args->q, (T*)args->k, (T*)args->v, (const T*)args->bias, nullptr,
+                                  (int)args->seq, (int)args->heads, (int)args->head_dim, hidden,
+                                  FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim)};
+        return (launch_gemm<T, false>(g, epi, 1, aligned, s));
+      }
+      default:
+        return fail(TTMI_EINVAL, "unknown epilogue");
+    }
+  });
+  return 0;
+}
+
+int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_t n, int64_t k, int64_t lda,
+                 int64_t ldb, int64_t ldc, void* stream) {
+  TTMI_REQUIRE(a && b && c, "null matrix");
+  TTMI_REQUIRE(m < (1ll << 31) && n < (1ll << 31) && k < (1ll << 31), "dimension too large");
+  TTMI_REQUIRE(lda >= k && ldb >= k && ldc >= n, "leading dimension too small");
+  GemmArgs g{};
+  g.a = (const char*)a;
+  g.b = (const char*)b;
+  g.m = (int)m; g.n = (int)n; g.k = (int)k;
+  g.lda = lda; g.ldb = ldb;
+  g.inner = 1;
+  EpiInt32 epi{c, ldc};
+  const bool aligned = aligned16(a) && aligned16(b) && lda % 16 == 0 && ldb % 16 == 0 && k % 16 == 0;
+  return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
+}
+
+}  // extern "C"

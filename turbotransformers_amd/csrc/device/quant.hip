@@ -1,0 +1,107 @@
+// Small kernels around the int8 GEMM (dynamic per-tensor activation quantisation and the
+// fp32 dequant+bias epilogue) and the per-token row map of a packed (smart) batch.
+#include "common.h"
+
+namespace ttmi {
+
+// |x| as uint bits orders like the float for non-negative values, so one integer
+// atomicMax per block yields max|x|.
+__global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ x, int64_t n,
+                                                     uint32_t* __restrict__ out_bits) {
+  __shared__ float red[4];
+  float mx = 0.f;
+  int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i < n; i += stride) mx = fmaxf(mx, fabsf(x[i]));
+  mx = group_max<kWave>(mx);
+  if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    atomicMax(out_bits, __float_as_uint(mx));
+  }
+}
+
+__global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, int8_t* __restrict__ q,
+                                                       float* __restrict__ scale_dev, int64_t n) {
+  const float mx = scale_dev[1];
+  const float scale = mx > 0.f ? mx / 127.0f : 1.0f;
+  int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  if (i == 0) scale_dev[0] = scale;
+  for (; i < n; i += stride) {
+    float r = rintf(x[i] / scale);  // round half to even
+    r = fminf(fmaxf(r, -127.f), 127.f);
+    q[i] = (int8_t)r;
+  }
+}
+
+__global__ __launch_bounds__(256) void dequant_bias_kernel(const int32_t* __restrict__ acc,
+                                                           const float* __restrict__ act_scale,
+                                                           const float* __restrict__ w_scale,
+                                                           const float* __restrict__ bias,
+                                                           float* __restrict__ out, int64_t total, int n) {
+  const float sx = act_scale[0];
+  int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i < total; i += stride) {
+    const int c = (int)(i % n);
+    float v = (float)acc[i] * sx * w_scale[c];
+    if (bias) v += bias[c];
+    out[i] = v;
+  }
+}
+
+__global__ void token_rows_kernel(const int32_t* __restrict__ cu, int batch, int max_seq, int total,
+                                  int32_t* __restrict__ rows) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= total) return;
+  int lo = 0, hi = batch;  // find b with cu[b] <= t < cu[b+1]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  rows[t] = lo * max_seq + (t - cu[lo]);
+}
+
+static unsigned flat_grid(int64_t n) { return (unsigned)std::min<int64_t>(ceil_div(n, 256), 256 * 16); }
+
+}  // namespace ttmi
+
+using namespace ttmi;
+
+extern "C" {
+
+int ttmi_quantize_rows_i8(const float* x, int8_t* q, float* scale_dev, int64_t m, int64_t k, void* stream) {
+  TTMI_REQUIRE(x && q && scale_dev, "null tensor");
+  const int64_t n = m * k;
+  if (n <= 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  int rc = ttmi_memset_zero(scale_dev, 2 * sizeof(float), stream);
+  if (rc != 0) return rc;
+  hipLaunchKernelGGL(absmax_kernel, dim3(flat_grid(n)), dim3(256), 0, s, x, n, reinterpret_cast<uint32_t*>(scale_dev + 1));
+  hipLaunchKernelGGL(quantize_kernel, dim3(flat_grid(n)), dim3(256), 0, s, x, q, scale_dev, n);
+  return launch_status("quantize_rows_i8");
+}
+
+int ttmi_dequant_bias(const int32_t* acc, const float* act_scale_dev, const float* w_scale, const float* bias,
+                      float* out, int64_t m, int64_t n, void* stream) {
+  TTMI_REQUIRE(acc && act_scale_dev && w_scale && out, "null tensor");
+  TTMI_REQUIRE(n < (1ll << 31), "N too large");
+  if (m * n <= 0) return 0;
+  hipLaunchKernelGGL(dequant_bias_kernel, dim3(flat_grid(m * n)), dim3(256), 0, (hipStream_t)stream, acc,
+                     act_scale_dev, w_scale, bias, out, m * n, (int)n);
+  return launch_status("dequant_bias");
+}
+
+int ttmi_build_token_rows(const int32_t* cu_seqlens, int64_t batch, int64_t max_seq, int64_t total,
+                          int32_t* token_rows, void* stream) {
+  TTMI_REQUIRE(cu_seqlens && token_rows, "null tensor");
+  TTMI_REQUIRE(batch > 0 && batch * max_seq < (1ll << 31) && total < (1ll << 31), "bad shape");
+  if (total <= 0) return 0;
+  hipLaunchKernelGGL(token_rows_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, (hipStream_t)stream,
+                     cu_seqlens, (int)batch, (int)max_seq, (int)total, token_rows);
+  return launch_status("build_token_rows");
+}
+
+}  // extern "C"

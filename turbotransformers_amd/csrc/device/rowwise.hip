@@ -1,0 +1,360 @@
+// Row-wise, HBM-bound kernels: LayerNorm / AddBiasLayerNorm and ApplyMaskAndSoftmax.
+//
+// Layout idea shared by both: a row is owned by a group of G lanes of one wavefront
+// (G = 8..64); every lane keeps ITERS 16-byte vectors of the row in registers, so the row
+// is read from HBM once and written once, and the two reductions are wave64 shuffles with
+// no LDS and no block barrier.  A block is 256 threads = 4 wavefronts = 256/G rows.
+// Rows too long for the register budget go to a block-per-row fallback.
+#include "common.h"
+
+namespace ttmi {
+
+constexpr int kBlock = 256;
+
+// --------------------------------------------------------------------------- LayerNorm --
+// x = out (+ input + bias); mean = sum(x)/n; var = sum(x*x)/n - mean^2;
+// out = beta + gamma * (x - mean) * rsqrt(var + eps)      (layer_norm.cpp:144-163)
+template <typename T, int VEC, int G, int ITERS, bool ADD>
+__global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, const T* __restrict__ input,
+                                                          const T* __restrict__ bias,
+                                                          const T* __restrict__ gamma,
+                                                          const T* __restrict__ beta, int64_t m, int n,
+                                                          float eps) {
+  constexpr int ROWS = kBlock / G;
+  const int lane = threadIdx.x % G;
+  const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / G;
+  const bool row_ok = row < m;
+  T* orow = out + row * n;
+  const T* irow = ADD ? input + row * n : nullptr;
+
+  float x[ITERS][VEC];
+  float sum = 0.f, sumsq = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int col = (it * G + lane) * VEC;
+    if (row_ok && col < n) {
+      Vec<T, VEC> o = load_vec<T, VEC>(orow + col);
+      if (ADD) {
+        Vec<T, VEC> a = load_vec<T, VEC>(irow + col);
+        Vec<T, VEC> b = load_vec<T, VEC>(bias + col);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[it][j] = to_float(o.v[j]) + to_float(a.v[j]) + to_float(b.v[j]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[it][j] = to_float(o.v[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        sum += x[it][j];
+        sumsq += x[it][j] * x[it][j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) x[it][j] = 0.f;
+    }
+  }
+  sum = group_sum<G>(sum);
+  sumsq = group_sum<G>(sumsq);
+  const float mean = sum / (float)n;
+  const float var = sumsq / (float)n - mean * mean;
+  const float rstd = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int col = (it * G + lane) * VEC;
+    if (row_ok && col < n) {
+      Vec<T, VEC> g = load_vec<T, VEC>(gamma + col);
+      Vec<T, VEC> b = load_vec<T, VEC>(beta + col);
+      Vec<T, VEC> o;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j)
+        o.v[j] = from_float<T>(to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean));
+      store_vec<T, VEC>(orow + col, o);
+    }
+  }
+}
+
+// Fallback: one block per row, any n; the row is re-read from L2 for the second pass.
+template <typename T, bool ADD>
+__global__ __launch_bounds__(kBlock) void layer_norm_block(T* __restrict__ out, const T* __restrict__ input,
+                                                           const T* __restrict__ bias,
+                                                           const T* __restrict__ gamma,
+                                                           const T* __restrict__ beta, int64_t m, int n,
+                                                           float eps) {
+  __shared__ float red[2][kBlock / kWave];
+  const int64_t row = blockIdx.x;
+  T* orow = out + row * n;
+  const T* irow = ADD ? input + row * n : nullptr;
+  float sum = 0.f, sumsq = 0.f;
+  for (int c = threadIdx.x; c < n; c += kBlock) {
+    float x = to_float(orow[c]);
+    if (ADD) x = x + to_float(irow[c]) + to_float(bias[c]);
+    sum += x;
+    sumsq += x * x;
+  }
+  sum = group_sum<kWave>(sum);
+  sumsq = group_sum<kWave>(sumsq);
+  if (threadIdx.x % kWave == 0) {
+    red[0][threadIdx.x / kWave] = sum;
+    red[1][threadIdx.x / kWave] = sumsq;
+  }
+  __syncthreads();
+  sum = 0.f;
+  sumsq = 0.f;
+#pragma unroll
+  for (int w = 0; w < kBlock / kWave; ++w) {
+    sum += red[0][w];
+    sumsq += red[1][w];
+  }
+  const float mean = sum / (float)n;
+  const float var = sumsq / (float)n - mean * mean;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  for (int c = threadIdx.x; c < n; c += kBlock) {
+    float x = to_float(orow[c]);
+    if (ADD) x = x + to_float(irow[c]) + to_float(bias[c]);
+    orow[c] = from_float<T>(to_float(beta[c]) + to_float(gamma[c]) * rstd * (x - mean));
+  }
+}
+
+template <typename T, int VEC, int G, int ITERS, bool ADD>
+static int launch_ln_rows(T* out, const T* input, const T* bias, const T* gamma, const T* beta, int64_t m,
+                          int n, float eps, hipStream_t s) {
+  constexpr int ROWS = kBlock / G;
+  const int64_t grid = ceil_div(m, ROWS);
+  hipLaunchKernelGGL((layer_norm_rows<T, VEC, G, ITERS, ADD>), dim3((unsigned)grid), dim3(kBlock), 0, s, out,
+                     input, bias, gamma, beta, m, n, eps);
+  return launch_status("layer_norm_rows");
+}
+
+template <typename T, bool ADD>
+static int layer_norm_dispatch(T* out, const T* input, const T* bias, const T* gamma, const T* beta,
+                               int64_t m, int64_t n, float eps, hipStream_t s) {
+  if (m == 0 || n == 0) return 0;
+  constexpr int VEC = 16 / sizeof(T);
+  auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool vec_ok = (n % VEC == 0) && aligned16(out) && aligned16(gamma) && aligned16(beta) &&
+                      (!ADD || (aligned16(input) && aligned16(bias)));
+  if (vec_ok) {
+    const int64_t nv = n / VEC;  // 16-byte vectors per row
+    // Pick the group width G so that nv = G * ITERS with as little idle lane time as possible.
+#define TTMI_LN_CASE(G, ITERS) return launch_ln_rows<T, VEC, G, ITERS, ADD>(out, input, bias, gamma, beta, m, (int)n, eps, s)
+    if (nv <= 16) TTMI_LN_CASE(16, 1);
+    if (nv <= 32) TTMI_LN_CASE(32, 1);
+    if (nv <= 64) TTMI_LN_CASE(64, 1);
+    if (nv <= 96 && nv % 32 == 0) TTMI_LN_CASE(32, 3);  // H=768 fp16/bf16
+    if (nv <= 128) TTMI_LN_CASE(64, 2);
+    if (nv <= 192) TTMI_LN_CASE(64, 3);                 // H=768 fp32
+    if (nv <= 256) TTMI_LN_CASE(64, 4);                 // H=1024 fp32
+    if (nv <= 384) TTMI_LN_CASE(64, 6);
+    if (nv <= 512) TTMI_LN_CASE(64, 8);
+#undef TTMI_LN_CASE
+  }
+  TTMI_REQUIRE(m < (1ll << 31), "too many rows");
+  hipLaunchKernelGGL((layer_norm_block<T, ADD>), dim3((unsigned)m), dim3(kBlock), 0, s, out, input, bias,
+                     gamma, beta, m, (int)n, eps);
+  return launch_status("layer_norm_block");
+}
+
+// ----------------------------------------------------------------------------- softmax --
+// x = score*scale + mask; p = exp(x - max) * (1/sum)        (softmax.cpp:28-81)
+template <typename T, int VEC, int G, int ITERS>
+__global__ __launch_bounds__(kBlock) void softmax_rows(T* __restrict__ score, const float* __restrict__ mask,
+                                                       int64_t rows, int heads, int from_len, int to_len,
+                                                       int mask_is_2d, float scale) {
+  constexpr int ROWS = kBlock / G;
+  const int lane = threadIdx.x % G;
+  const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / G;
+  const bool row_ok = row < rows;
+  T* srow = score + row * to_len;
+  const float* mrow = nullptr;
+  if (mask != nullptr && row_ok) {
+    const int64_t b = row / ((int64_t)heads * from_len);
+    const int64_t f = row % from_len;
+    mrow = mask + (mask_is_2d ? b * to_len : (b * from_len + f) * to_len);
+  }
+  float x[ITERS][VEC];
+  float mx = -3.402823466e+38f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int col = (it * G + lane) * VEC;
+    if (row_ok && col < to_len) {
+      Vec<T, VEC> s = load_vec<T, VEC>(srow + col);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        float v = to_float(s.v[j]) * scale;
+        if (mrow) v += mrow[col + j];
+        x[it][j] = v;
+        mx = fmaxf(mx, v);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) x[it][j] = -3.402823466e+38f;
+    }
+  }
+  mx = group_max<G>(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int col = (it * G + lane) * VEC;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float e = (row_ok && col < to_len) ? __expf(x[it][j] - mx) : 0.f;
+      x[it][j] = e;
+      sum += e;
+    }
+  }
+  sum = group_sum<G>(sum);
+  const float coef = 1.0f / sum;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int col = (it * G + lane) * VEC;
+    if (row_ok && col < to_len) {
+      Vec<T, VEC> o;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(x[it][j] * coef);
+      store_vec<T, VEC>(srow + col, o);
+    }
+  }
+}
+
+// Fallback for very long rows: block per row, three passes over L2-resident data.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void softmax_block(T* __restrict__ score, const float* __restrict__ mask,
+                                                        int64_t rows, int heads, int from_len, int to_len,
+                                                        int mask_is_2d, float scale) {
+  __shared__ float red[kBlock / kWave];
+  const int64_t row = blockIdx.x;
+  T* srow = score + row * to_len;
+  const float* mrow = nullptr;
+  if (mask != nullptr) {
+    const int64_t b = row / ((int64_t)heads * from_len);
+    const int64_t f = row % from_len;
+    mrow = mask + (mask_is_2d ? b * to_len : (b * from_len + f) * to_len);
+  }
+  float mx = -3.402823466e+38f;
+  for (int c = threadIdx.x; c < to_len; c += kBlock) {
+    float v = to_float(srow[c]) * scale;
+    if (mrow) v += mrow[c];
+    mx = fmaxf(mx, v);
+  }
+  mx = group_max<kWave>(mx);
+  if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = mx;
+  __syncthreads();
+  mx = red[0];
+#pragma unroll
+  for (int w = 1; w < kBlock / kWave; ++w) mx = fmaxf(mx, red[w]);
+  __syncthreads();
+  float sum = 0.f;
+  for (int c = threadIdx.x; c < to_len; c += kBlock) {
+    float v = to_float(srow[c]) * scale;
+    if (mrow) v += mrow[c];
+    sum += __expf(v - mx);
+  }
+  sum = group_sum<kWave>(sum);
+  if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = sum;
+  __syncthreads();
+  sum = 0.f;
+#pragma unroll
+  for (int w = 0; w < kBlock / kWave; ++w) sum += red[w];
+  const float coef = 1.0f / sum;
+  for (int c = threadIdx.x; c < to_len; c += kBlock) {
+    float v = to_float(srow[c]) * scale;
+    if (mrow) v += mrow[c];
+    srow[c] = from_float<T>(__expf(v - mx) * coef);
+  }
+}
+
+template <typename T, int VEC, int G, int ITERS>
+static int launch_softmax_rows(T* score, const float* mask, int64_t rows, int heads, int from_len, int to_len,
+                               int mask_is_2d, float scale, hipStream_t s) {
+  constexpr int ROWS = kBlock / G;
+  hipLaunchKernelGGL((softmax_rows<T, VEC, G, ITERS>), dim3((unsigned)ceil_div(rows, ROWS)), dim3(kBlock), 0,
+                     s, score, mask, rows, heads, from_len, to_len, mask_is_2d, scale);
+  return launch_status("softmax_rows");
+}
+
+template <typename T, int VEC>
+static int softmax_vec_dispatch(T* score, const float* mask, int64_t rows, int heads, int from_len, int to_len,
+                                int mask_is_2d, float scale, hipStream_t s, bool* done) {
+  const int nv = (to_len + VEC - 1) / VEC;
+  *done = true;
+#define TTMI_SM_CASE(G, ITERS) \
+  return launch_softmax_rows<T, VEC, G, ITERS>(score, mask, rows, heads, from_len, to_len, mask_is_2d, scale, s)
+  if (nv <= 8) TTMI_SM_CASE(8, 1);
+  if (nv <= 16) TTMI_SM_CASE(16, 1);
+  if (nv <= 32) TTMI_SM_CASE(32, 1);
+  if (nv <= 64) TTMI_SM_CASE(64, 1);
+  if (nv <= 128) TTMI_SM_CASE(64, 2);
+  if (nv <= 256) TTMI_SM_CASE(64, 4);
+  if (nv <= 512) TTMI_SM_CASE(64, 8);
+  if (nv <= 1024) TTMI_SM_CASE(64, 16);
+#undef TTMI_SM_CASE
+  *done = false;
+  return 0;
+}
+
+template <typename T>
+static int softmax_dispatch(T* score, const float* mask, int64_t batch, int64_t heads, int64_t from_len,
+                            int64_t to_len, int mask_is_2d, float scale, hipStream_t s) {
+  const int64_t rows = batch * heads * from_len;
+  if (rows == 0 || to_len == 0) return 0;
+  TTMI_REQUIRE(to_len < (1ll << 30) && from_len < (1ll << 30) && heads < (1ll << 30), "dimension too large");
+  constexpr int VMAX = 16 / sizeof(T);
+  // Row starts are row*to_len elements from a 16-byte aligned base: pick the widest vector
+  // that divides to_len so every row start stays aligned for it.
+  const bool base_ok = (reinterpret_cast<uintptr_t>(score) & 15) == 0;
+  int vec = 1;
+  if (base_ok) {
+    vec = VMAX;
+    while (vec > 1 && (to_len % vec) != 0) vec >>= 1;
+  }
+  bool done = false;
+  int rc = 0;
+  switch (vec) {
+    case 8: if constexpr (VMAX >= 8) { rc = softmax_vec_dispatch<T, 8>(score, mask, rows, (int)heads, (int)from_len, (int)to_len, mask_is_2d, scale, s, &done); } break;
+    case 4: rc = softmax_vec_dispatch<T, 4>(score, mask, rows, (int)heads, (int)from_len, (int)to_len, mask_is_2d, scale, s, &done); break;
+    case 2: rc = softmax_vec_dispatch<T, 2>(score, mask, rows, (int)heads, (int)from_len, (int)to_len, mask_is_2d, scale, s, &done); break;
+    default: rc = softmax_vec_dispatch<T, 1>(score, mask, rows, (int)heads, (int)from_len, (int)to_len, mask_is_2d, scale, s, &done); break;
+  }
+  if (done) return rc;
+  TTMI_REQUIRE(rows < (1ll << 31), "too many rows");
+  hipLaunchKernelGGL((softmax_block<T>), dim3((unsigned)rows), dim3(kBlock), 0, s, score, mask, rows,
+                     (int)heads, (int)from_len, (int)to_len, mask_is_2d, scale);
+  return launch_status("softmax_block");
+}
+
+}  // namespace ttmi
+
+using namespace ttmi;
+
+extern "C" {
+
+int ttmi_layer_norm(void* out, const void* gamma, const void* beta, int64_t m, int64_t n, float eps, int dtype,
+                    void* stream) {
+  TTMI_REQUIRE(out && gamma && beta, "null tensor");
+  TTMI_REQUIRE(m >= 0 && n >= 0 && n < (1ll << 31), "bad shape");
+  TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, false>((T*)out, nullptr, nullptr, (const T*)gamma,
+                                                                       (const T*)beta, m, n, eps,
+                                                                       (hipStream_t)stream)));
+  return 0;
+}
+
+int ttmi_add_bias_layer_norm(void* out, const void* input, const void* bias, const void* gamma,
+                             const void* beta, int64_t m, int64_t n, float eps, int dtype, void* stream) {
+  TTMI_REQUIRE(out && input && bias && gamma && beta, "null tensor");
+  TTMI_REQUIRE(m >= 0 && n >= 0 && n < (1ll << 31), "bad shape");
+  TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, true>((T*)out, (const T*)input, (const T*)bias,
+                                                                      (const T*)gamma, (const T*)beta, m, n, eps,
+                                                                      (hipStream_t)stream)));
+  return 0;
+}
+
+int ttmi_apply_mask_and_softmax(void* score, const float* mask, int64_t batch, int64_t heads, int64_t from_len,
+                                int64_t to_len, int mask_is_2d, float scale, int dtype, void* stream) {
+  TTMI_REQUIRE(score != nullptr, "null score");
+  TTMI_REQUIRE(batch >= 0 && heads >= 0 && from_len >= 0 && to_len >= 0, "bad shape");
+  TTMI_DISPATCH_FLOAT(dtype, T, return softmax_dispatch<T>((T*)score, mask, batch, heads, from_len, to_len,
+                                                           mask_is_2d, scale, (hipStream_t)stream));
+  return 0;
+}
+
+}  // extern "C"

@@ -106,6 +106,14 @@ TTMI_API int ttmi_add_bias_layer_norm(void* out, const void* input, const void* 
                                       const void* beta, int64_t m, int64_t n, float eps, int dtype,
                                       void* stream);
 
+/* AddBiasLayerNorm whose residual stream stays in fp32 while `out` is 16-bit storage:
+ *   y = LN(out + residual_f32 + bias);  out = round(y);  out_f32 = y.
+ * residual_f32 and out_f32 may be the same buffer.  Used by the layers for bfloat16 models so
+ * that only GEMM operands are rounded (no counterpart in the reference, which is fp32-only). */
+TTMI_API int ttmi_add_bias_layer_norm_residual32(void* out, const float* residual_f32, const void* bias,
+                                                 const void* gamma, const void* beta, float* out_f32, int64_t m,
+                                                 int64_t n, float eps, int dtype, void* stream);
+
 /* kernels::AddBiasAct<T, Act>  (layers/kernels/activation.cpp:33-55, 90-119).
  * out[m,n] = act(out[m,n] + bias[n]) in place; gelu is the tanh form. */
 TTMI_API int ttmi_add_bias_act(void* out, const void* bias, int64_t m, int64_t n, int act, int dtype,
@@ -169,6 +177,13 @@ TTMI_API int ttmi_bert_embedding(void* out, const int64_t* ids, const int64_t* p
                                  const void* type_table, const void* gamma, const void* beta,
                                  int64_t num_ids, int64_t hidden, int64_t vocab, int64_t max_pos,
                                  int64_t num_types, float eps, int dtype, void* stream);
+/* Same, also writing the unrounded LayerNorm output to out_f32 (start of an fp32 residual stream). */
+TTMI_API int ttmi_bert_embedding_residual32(void* out, float* out_f32, const int64_t* ids, const int64_t* pos_ids,
+                                            const int64_t* type_ids, const void* word_table,
+                                            const void* pos_table, const void* type_table, const void* gamma,
+                                            const void* beta, int64_t num_ids, int64_t hidden, int64_t vocab,
+                                            int64_t max_pos, int64_t num_types, float eps, int dtype,
+                                            void* stream);
 
 /* kernels::common::Sequence / Fill / Transform  (layers/kernels/common.cpp:29-90), the three
  * helpers of layers::PrepareBertMasks (layers/prepare_bert_masks.cpp:24-66). */
@@ -178,6 +193,11 @@ TTMI_API int ttmi_fill_f32(float* data, int64_t n, float value, void* stream);
 TTMI_API int ttmi_sequence_rows_i64(int64_t* data, int64_t rows, int64_t cols, void* stream);
 /* dst[i] = -10000 * (1 - src[i]) */
 TTMI_API int ttmi_mask_transform(const int64_t* src, float* dst, int64_t n, void* stream);
+
+/* kernels::SeqPool  (layers/kernels/seq_pool.cpp:124-155): in[B,S,H] -> out[B,H];
+ * pool_type 0 = max, 1 = mean, 2 = first, 3 = last (layers/types.h PoolType order). */
+TTMI_API int ttmi_seq_pool(const void* in, void* out, int64_t batch, int64_t seq, int64_t hidden, int pool_type,
+                           int dtype, void* stream);
 
 /* Smart-batch key-padding mask (python layers/modeling_smart_pad.py:465-475):
  * mask[b, 0, t] = 0 for t < len[b] else -1e9, shape [B,1,max_seq] fp32. */

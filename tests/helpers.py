@@ -59,3 +59,26 @@ def ok(rc):
 
 def max_abs(a, b):
     return float(np.max(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)))) if np.size(a) else 0.0
+
+
+def oracle_layer_weights(w, prefix=""):
+    """HuggingFace parameter dict (numpy, names as in BertModel.named_parameters) -> the oracle's
+    per-layer weights, packed the way BertAttention.from_torch packs them: dense weights
+    transposed to [in, out], q/k/v concatenated along the output axis."""
+    g = lambda n: np.asarray(w[prefix + n], np.float32)
+    return {
+        "qkv_w": np.ascontiguousarray(np.concatenate([g("attention.self.query.weight"), g("attention.self.key.weight"),
+                                                      g("attention.self.value.weight")], 0).T),
+        "qkv_b": np.concatenate([g("attention.self.query.bias"), g("attention.self.key.bias"),
+                                 g("attention.self.value.bias")]),
+        "attn_out_w": np.ascontiguousarray(g("attention.output.dense.weight").T),
+        "attn_out_b": g("attention.output.dense.bias"),
+        "attn_ln_g": g("attention.output.LayerNorm.weight"),
+        "attn_ln_b": g("attention.output.LayerNorm.bias"),
+        "inter_w": np.ascontiguousarray(g("intermediate.dense.weight").T),
+        "inter_b": g("intermediate.dense.bias"),
+        "out_w": np.ascontiguousarray(g("output.dense.weight").T),
+        "out_b": g("output.dense.bias"),
+        "out_ln_g": g("output.LayerNorm.weight"),
+        "out_ln_b": g("output.LayerNorm.bias"),
+    }

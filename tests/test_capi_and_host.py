@@ -1,0 +1,132 @@
+"""CPU-side checks of the boundary: the C-ABI library loads and exports every symbol that
+include/ttmi.h declares, the pybind module and the drop-in package import, and the host
+logic that needs no GPU (Tensor/DLPack semantics, allocator rounding, the npz reader, error
+paths).  No compute entry point is called here.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+from turbotransformers_amd import capi
+
+
+def test_header_declares_and_library_exports_every_entry_point():
+    protos = capi.parse_header()
+    assert len(protos) >= 45
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    missing = [n for n in protos if not hasattr(lib, n)]
+    assert not missing, missing
+    # and nothing with C linkage is exported that the header does not declare
+    out = subprocess.run(["nm", "-D", "--defined-only", capi.LIB_PATH], capture_output=True, text=True).stdout
+    exported = {l.split()[-1] for l in out.splitlines() if " T " in l and l.split()[-1].startswith("ttmi_")}
+    assert exported == set(protos), exported ^ set(protos)
+
+
+def test_every_declaration_cites_or_explains_itself():
+    text = open(capi.HEADER).read()
+    assert text.count("TTMI_API int") >= 40 and "extern \"C\"" in text
+    assert "torch" not in text.split("*/", 1)[1].lower().replace("pytorch", "")  # no torch types in signatures
+
+
+def test_error_reporting_without_a_gpu():
+    lib = capi.load()
+    rc = lib.ttmi_layer_norm(None, None, None, 1, 8, 1e-12, capi.F32, None)
+    assert rc == -1 and b"null tensor" in lib.ttmi_last_error()
+    with pytest.raises(capi.TtmiError):
+        capi.check(lib.ttmi_gemm(None, None, None, 1, 1, 1, 1, 1, 1, 0, 1.0, 0.0, capi.F32, None))
+    n = ctypes.c_int(-1)
+    assert lib.ttmi_device_count(ctypes.byref(n)) == 0 and n.value >= 0
+
+
+def test_dropin_package_surface():
+    import turbo_transformers as tt
+    import turbo_transformers.turbo_transformers_cxx as cxx
+    for name in ("BertModel", "BertLayer", "BertEncoder", "BertAttention", "BertIntermediate", "BertOutput",
+                 "BertEmbeddings", "BertPooler", "SequencePool", "PoolingType", "ReturnType", "BertModelSmartBatch",
+                 "MultiHeadedAttentionSmartBatch", "AlbertModel", "AlbertLayer"):
+        assert hasattr(tt, name), name
+    for name in ("Tensor", "BERTEmbedding", "BertAttention", "MultiHeadedAttention", "MultiHeadedAttentionSmartBatch",
+                 "BertIntermediate", "BertOutput", "SequencePool", "BertPooler", "PrepareBertMasks", "AlbertLayer",
+                 "FusedAddBiasGELU", "FusedAddBiasLayerNorm", "nparray2tensor", "tensor2nparrayf", "tensor2nparrayl",
+                 "set_num_threads", "reset_allocator_schema", "bert_opt_mem_allocate_api", "enable_perf", "disable_perf",
+                 "set_stderr_verbose_level"):
+        assert hasattr(cxx, name), name
+    assert cxx.config.is_compiled_with_cuda() is True
+    assert callable(tt.BertModel.from_torch)
+
+
+def test_tensor_dlpack_round_trip_and_ownership():
+    import turbo_transformers.turbo_transformers_cxx as cxx
+    t = torch.arange(24, dtype=torch.float32).reshape(2, 3, 4)
+    capsule = torch.utils.dlpack.to_dlpack(t)
+    tt = cxx.Tensor.from_dlpack(capsule)
+    assert tt.n_dim() == 3 and [tt.shape(i) for i in range(3)] == [2, 3, 4] and tt.shape(-1) == 4
+    assert tt.float_data() == t.data_ptr()            # alias, not a copy
+    with pytest.raises(RuntimeError):
+        tt.shape(3)
+    back = torch.utils.dlpack.from_dlpack(tt.to_dlpack())
+    assert back.data_ptr() == t.data_ptr() and torch.equal(back, t)
+    assert tt.is_null()                               # to_dlpack released ownership
+    with pytest.raises(RuntimeError):
+        tt.to_dlpack()
+    assert cxx.Tensor.create_empty().is_null()
+    i64 = cxx.Tensor.from_dlpack(torch.utils.dlpack.to_dlpack(torch.ones(3, dtype=torch.int64)))
+    with pytest.raises(RuntimeError):                 # dtype check of data<float>()
+        i64.float_data()
+
+
+def test_numpy_converters_on_cpu():
+    import turbo_transformers.turbo_transformers_cxx as cxx
+    a = np.arange(12, dtype=np.float32).reshape(3, 4)
+    t = cxx.nparray2tensor(a, "CPU")
+    assert np.array_equal(cxx.tensor2nparrayf(t), a)
+    ids = np.arange(5, dtype=np.int64)
+    assert np.array_equal(cxx.tensor2nparrayl(cxx.nparray2tensor(ids, "CPU")), ids)
+    with pytest.raises(RuntimeError):
+        cxx.nparray2tensor(a, "TPU")
+
+
+def test_layers_reject_cpu_tensors_and_bad_shapes():
+    """No CPU fallback: a layer built on host tensors refuses to run; shape checks raise."""
+    import turbo_transformers.turbo_transformers_cxx as cxx
+    conv = lambda x: cxx.Tensor.from_dlpack(torch.utils.dlpack.to_dlpack(x))
+    inter = cxx.BertIntermediate(conv(torch.zeros(8, 32)), conv(torch.zeros(32)))
+    with pytest.raises(RuntimeError, match="not on the GPU"):
+        inter(conv(torch.zeros(2, 8)), cxx.Tensor.create_empty())
+    with pytest.raises(RuntimeError):  # weight/bias mismatch (bert_intermediate.cpp EnforceShapeAndType)
+        cxx.BertIntermediate(conv(torch.zeros(8, 32)), conv(torch.zeros(31)))
+    with pytest.raises(RuntimeError):
+        cxx.SequencePool("Median")
+    with pytest.raises(RuntimeError):
+        cxx.reset_allocator_schema("no-such-schema")
+    cxx.reset_allocator_schema("naive")
+    import turbo_transformers as tt
+    from transformers import BertConfig, BertModel
+    tiny = BertModel(BertConfig(vocab_size=10, hidden_size=8, num_hidden_layers=1, num_attention_heads=2,
+                                intermediate_size=16, max_position_embeddings=8))
+    with pytest.raises(RuntimeError, match="GPU"):
+        tt.BertModel.from_torch(tiny, torch.device("cpu"), "turbo")
+    with pytest.raises(NotImplementedError):
+        tt.BertModel.from_torch(tiny, torch.device("cpu"), "onnxrt")
+
+
+def test_npz_reader_matches_numpy(tmp_path):
+    import turbo_transformers.turbo_transformers_cxx as cxx
+    rng = np.random.default_rng(0)
+    arrays = {"embeddings.word_embeddings.weight": rng.standard_normal((7, 4)).astype(np.float32),
+              "pooler.dense.bias": rng.standard_normal(4).astype(np.float32),
+              "half": rng.standard_normal((2, 3)).astype(np.float16),
+              "ids": np.arange(6, dtype=np.int64).reshape(2, 3)}
+    path = str(tmp_path / "w.npz")
+    np.savez(path, **arrays)
+    loaded = cxx.load_npz(path)
+    assert set(loaded) == set(arrays)
+    for k, v in arrays.items():
+        assert loaded[k].dtype == v.dtype and np.array_equal(loaded[k], v)
+    np.savez_compressed(path, **arrays)
+    with pytest.raises(RuntimeError, match="compressed"):
+        cxx.load_npz(path)

@@ -31,6 +31,28 @@ def test_add_bias_layer_norm(ttmi, oracle, dt, m, n):
     assert max_abs(host(d_out), want) <= TOL[dt] * 4
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("m,n", [(37, 768), (8, 1024), (5, 770)])
+def test_add_bias_layer_norm_fp32_residual(ttmi, oracle, dt, m, n):
+    """16-bit GEMM output + fp32 residual stream: the fp32 result equals the oracle on the same
+    values to fp32 accuracy, and the 16-bit output is its rounding."""
+    rng = np.random.default_rng(n)
+    out, res = rng.standard_normal((m, n), np.float32), rng.standard_normal((m, n), np.float32)
+    bias, gamma, beta = (rng.standard_normal(n).astype(np.float32) for _ in range(3))
+    d_out, d_res = dev(out, dt), dev(res)
+    d_out32 = torch.empty((m, n), device="cuda")
+    ok(ttmi.ttmi_add_bias_layer_norm_residual32(ptr(d_out), ptr(d_res), ptr(dev(bias, dt)), ptr(dev(gamma, dt)),
+                                                ptr(dev(beta, dt)), ptr(d_out32), m, n, 1e-12, TTMI_DTYPES[dt], stream()))
+    want = oracle.add_bias_layer_norm(rounded(out, dt), res, rounded(bias, dt), rounded(gamma, dt), rounded(beta, dt))
+    assert max_abs(host(d_out32), want) <= 1e-4
+    assert np.array_equal(host(d_out), rounded(host(d_out32), dt))
+    # in place on the residual buffer
+    d_out = dev(out, dt)
+    ok(ttmi.ttmi_add_bias_layer_norm_residual32(ptr(d_out), ptr(d_res), ptr(dev(bias, dt)), ptr(dev(gamma, dt)),
+                                                ptr(dev(beta, dt)), ptr(d_res), m, n, 1e-12, TTMI_DTYPES[dt], stream()))
+    assert max_abs(host(d_res), want) <= 1e-4
+
+
 @pytest.mark.parametrize("dt", ALL_DTYPES)
 @pytest.mark.parametrize("m,n", [(20, 768), (9, 2000), (4, 100)])
 def test_layer_norm(ttmi, oracle, dt, m, n):

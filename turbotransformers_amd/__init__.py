@@ -1,0 +1,28 @@
+"""MI355X-native TurboTransformers BERT encoder path.
+
+`import turbotransformers_amd as turbo_transformers` (or the `turbo_transformers` alias
+package at the repository root) gives the reference's Python surface for this path:
+`BertModel.from_torch(...)`, the layer classes, `ReturnType`, `PoolingType`.
+
+Importing requires the two in-tree native libraries (libttmi.so, turbo_transformers_cxx);
+there is no Python or CPU fallback.
+"""
+import os as _os
+
+_here = _os.path.dirname(_os.path.abspath(__file__))
+try:
+    from . import turbo_transformers_cxx as cxx
+except ImportError as _e:  # fail loudly: nothing works without the native module
+    raise ImportError("turbo_transformers_cxx is not built (%s); run `python -m turbotransformers_amd.build`" % _e)
+
+from .layers import *  # noqa: E402,F401,F403
+from .layers import __all__ as _layers_all  # noqa: E402
+
+config = cxx.config
+set_num_threads = cxx.set_num_threads
+reset_allocator_schema = cxx.reset_allocator_schema
+bert_opt_mem_allocate_api = cxx.bert_opt_mem_allocate_api
+set_stderr_verbose_level = cxx.set_stderr_verbose_level
+
+__all__ = list(_layers_all) + ['cxx', 'config', 'set_num_threads', 'reset_allocator_schema',
+                                'bert_opt_mem_allocate_api', 'set_stderr_verbose_level']

@@ -47,15 +47,28 @@ def host_module_path():
     return os.path.join(PKG_DIR, "turbo_transformers_cxx" + ext)
 
 
-def build_device(jobs=8, verbose=True):
+def _stale(obj, sources):
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    return any(os.path.getmtime(s) > t for s in sources)
+
+
+def build_device(jobs=8, verbose=True, force=True):
+    """force=False recompiles only objects older than their source or any header."""
     src_dir = os.path.join(CSRC, "device")
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(OBJ_DIR, exist_ok=True)
     sources = sorted(f for f in os.listdir(src_dir) if f.endswith(".hip"))
     objs = []
 
+    headers = [os.path.join(src_dir, f) for f in os.listdir(src_dir) if f.endswith(".h")]
+    headers.append(os.path.join(INCLUDE, "ttmi.h"))
+
     def compile_one(name):
         obj = os.path.join(OBJ_DIR, name[:-4] + ".o")
+        if not force and not _stale(obj, [os.path.join(src_dir, name)] + headers):
+            return obj
         out = _run([HIPCC] + DEVICE_FLAGS + ["-c", os.path.join(src_dir, name), "-o", obj])
         if verbose and out.strip():
             print(out)
@@ -105,9 +118,8 @@ def build_all(verbose=True):
 
 if __name__ == "__main__":
     what = sys.argv[1] if len(sys.argv) > 1 else "all"
-    if what == "device":
-        build_device()
-    elif what == "host":
+    incremental = "--incremental" in sys.argv
+    if what in ("device", "all"):
+        build_device(force=not incremental)
+    if what in ("host", "all"):
         build_host()
-    else:
-        build_all()

@@ -192,7 +192,8 @@ __global__ __launch_bounds__(kBlock) void bert_embedding_kernel(
     T* __restrict__ out, const int64_t* __restrict__ ids, const int64_t* __restrict__ pos_ids,
     const int64_t* __restrict__ type_ids, const T* __restrict__ word, const T* __restrict__ pos,
     const T* __restrict__ type, const T* __restrict__ gamma, const T* __restrict__ beta, int64_t num_ids,
-    int hidden, int64_t vocab, int64_t max_pos, int64_t num_types, float eps, int* __restrict__ err) {
+    int hidden, int64_t vocab, int64_t max_pos, int64_t num_types, float eps, int* __restrict__ err,
+    float* __restrict__ out32) {
   const int lane = threadIdx.x % kWave;
   const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   if (row >= num_ids) return;  // whole wavefront exits together
@@ -240,8 +241,11 @@ __global__ __launch_bounds__(kBlock) void bert_embedding_kernel(
       Vec<T, VEC> b = load_vec<T, VEC>(beta + col);
       Vec<T, VEC> o;
 #pragma unroll
-      for (int j = 0; j < VEC; ++j)
-        o.v[j] = from_float<T>(to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean));
+      for (int j = 0; j < VEC; ++j) {
+        const float y = to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean);
+        o.v[j] = from_float<T>(y);
+        if (out32) out32[row * hidden + col + j] = y;
+      }
       store_vec<T, VEC>(orow + col, o);
     }
   }
@@ -293,7 +297,7 @@ template <typename T>
 static int bert_embedding_dispatch(T* out, const int64_t* ids, const int64_t* pos_ids, const int64_t* type_ids,
                                    const T* word, const T* pos, const T* type, const T* gamma, const T* beta,
                                    int64_t num_ids, int64_t hidden, int64_t vocab, int64_t max_pos,
-                                   int64_t num_types, float eps, hipStream_t s) {
+                                   int64_t num_types, float eps, hipStream_t s, float* out32 = nullptr) {
   int* err = async_error_flag();
   TTMI_REQUIRE(err != nullptr, "no async error flag");
   constexpr int VMAX = 16 / sizeof(T);
@@ -309,13 +313,37 @@ static int bert_embedding_dispatch(T* out, const int64_t* ids, const int64_t* po
     constexpr int ITERS = decltype(iters)::value;
     hipLaunchKernelGGL((bert_embedding_kernel<T, VMAX, ITERS>), grid, dim3(kBlock), 0, s, out, ids, pos_ids,
                        type_ids, word, pos, type, gamma, beta, num_ids, (int)hidden, vocab, max_pos, num_types, eps,
-                       err);
+                       err, out32);
   };
   if (nv <= 64) launch(std::integral_constant<int, 1>{});
   else if (nv <= 128) launch(std::integral_constant<int, 2>{});
   else if (nv <= 256) launch(std::integral_constant<int, 4>{});
   else launch(std::integral_constant<int, 8>{});
   return launch_status("bert_embedding");
+}
+
+// [B,S,H] -> [B,H]; type 0 max, 1 mean, 2 first, 3 last                 (seq_pool.cpp:124-155)
+template <typename T>
+__global__ void seq_pool_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t batch, int64_t seq,
+                                int64_t hidden, int type) {
+  const int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= batch * hidden) return;
+  const int64_t b = i / hidden, c = i % hidden;
+  const T* col = in + b * seq * hidden + c;
+  float r;
+  if (type == 2) {
+    r = to_float(col[0]);
+  } else if (type == 3) {
+    r = to_float(col[(seq - 1) * hidden]);
+  } else if (type == 1) {
+    r = 0.f;
+    for (int64_t s = 0; s < seq; ++s) r += to_float(col[s * hidden]);
+    r /= (float)seq;
+  } else {
+    r = to_float(col[0]);
+    for (int64_t s = 1; s < seq; ++s) r = fmaxf(r, to_float(col[s * hidden]));
+  }
+  out[i] = from_float<T>(r);
 }
 
 static unsigned flat_grid(int64_t n) { return (unsigned)std::min<int64_t>(ceil_div(n, 256), 256 * 16); }
@@ -431,6 +459,34 @@ int ttmi_bert_embedding(void* out, const int64_t* ids, const int64_t* pos_ids, c
                                                                   (const T*)beta, num_ids, hidden, vocab, max_pos,
                                                                   num_types, eps, (hipStream_t)stream));
   return 0;
+}
+
+int ttmi_bert_embedding_residual32(void* out, float* out_f32, const int64_t* ids, const int64_t* pos_ids,
+                                   const int64_t* type_ids, const void* word_table, const void* pos_table,
+                                   const void* type_table, const void* gamma, const void* beta, int64_t num_ids,
+                                   int64_t hidden, int64_t vocab, int64_t max_pos, int64_t num_types, float eps,
+                                   int dtype, void* stream) {
+  TTMI_REQUIRE(out && out_f32 && ids && pos_ids && type_ids && word_table && pos_table && type_table && gamma && beta,
+               "null tensor");
+  if (num_ids == 0) return 0;
+  TTMI_DISPATCH_FLOAT(dtype, T, return bert_embedding_dispatch<T>((T*)out, ids, pos_ids, type_ids,
+                                                                  (const T*)word_table, (const T*)pos_table,
+                                                                  (const T*)type_table, (const T*)gamma,
+                                                                  (const T*)beta, num_ids, hidden, vocab, max_pos,
+                                                                  num_types, eps, (hipStream_t)stream, out_f32));
+  return 0;
+}
+
+int ttmi_seq_pool(const void* in, void* out, int64_t batch, int64_t seq, int64_t hidden, int pool_type, int dtype,
+                  void* stream) {
+  TTMI_REQUIRE(in && out, "null tensor");
+  TTMI_REQUIRE(pool_type >= 0 && pool_type <= 3, "unknown pool type");
+  TTMI_REQUIRE(seq > 0, "sequence length must be positive");
+  if (batch * hidden <= 0) return 0;
+  const dim3 grid((unsigned)ceil_div(batch * hidden, 256));
+  TTMI_DISPATCH_FLOAT(dtype, T, hipLaunchKernelGGL((seq_pool_kernel<T>), grid, dim3(256), 0, (hipStream_t)stream,
+                                                   (const T*)in, (T*)out, batch, seq, hidden, pool_type));
+  return launch_status("seq_pool");
 }
 
 int ttmi_sequence_rows_i64(int64_t* data, int64_t rows, int64_t cols, void* stream) {

@@ -14,18 +14,22 @@ constexpr int kBlock = 256;
 // --------------------------------------------------------------------------- LayerNorm --
 // x = out (+ input + bias); mean = sum(x)/n; var = sum(x*x)/n - mean^2;
 // out = beta + gamma * (x - mean) * rsqrt(var + eps)      (layer_norm.cpp:144-163)
-template <typename T, int VEC, int G, int ITERS, bool ADD>
+//
+// RES32: the residual is read from an fp32 copy (`res32`) instead of `input`, and the result is
+// also written unrounded to `out32`.  With 16-bit storage this keeps the residual stream of the
+// encoder in fp32 -- only GEMM operands are rounded -- at the cost of 12 instead of 6 bytes/element.
+template <typename T, int VEC, int G, int ITERS, bool ADD, bool RES32>
 __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, const T* __restrict__ input,
                                                           const T* __restrict__ bias,
                                                           const T* __restrict__ gamma,
                                                           const T* __restrict__ beta, int64_t m, int n,
-                                                          float eps) {
+                                                          float eps, const float* res32, float* out32) {
   constexpr int ROWS = kBlock / G;
   const int lane = threadIdx.x % G;
   const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / G;
   const bool row_ok = row < m;
   T* orow = out + row * n;
-  const T* irow = ADD ? input + row * n : nullptr;
+  const T* irow = (ADD && !RES32) ? input + row * n : nullptr;
 
   float x[ITERS][VEC];
   float sum = 0.f, sumsq = 0.f;
@@ -34,7 +38,11 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
     const int col = (it * G + lane) * VEC;
     if (row_ok && col < n) {
       Vec<T, VEC> o = load_vec<T, VEC>(orow + col);
-      if (ADD) {
+      if (ADD && RES32) {
+        Vec<T, VEC> b = load_vec<T, VEC>(bias + col);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[it][j] = to_float(o.v[j]) + res32[row * n + col + j] + to_float(b.v[j]);
+      } else if (ADD) {
         Vec<T, VEC> a = load_vec<T, VEC>(irow + col);
         Vec<T, VEC> b = load_vec<T, VEC>(bias + col);
 #pragma unroll
@@ -66,28 +74,32 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
       Vec<T, VEC> b = load_vec<T, VEC>(beta + col);
       Vec<T, VEC> o;
 #pragma unroll
-      for (int j = 0; j < VEC; ++j)
-        o.v[j] = from_float<T>(to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean));
+      for (int j = 0; j < VEC; ++j) {
+        const float y = to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean);
+        o.v[j] = from_float<T>(y);
+        if (RES32) out32[row * n + col + j] = y;
+      }
       store_vec<T, VEC>(orow + col, o);
     }
   }
 }
 
 // Fallback: one block per row, any n; the row is re-read from L2 for the second pass.
-template <typename T, bool ADD>
+template <typename T, bool ADD, bool RES32>
 __global__ __launch_bounds__(kBlock) void layer_norm_block(T* __restrict__ out, const T* __restrict__ input,
                                                            const T* __restrict__ bias,
                                                            const T* __restrict__ gamma,
                                                            const T* __restrict__ beta, int64_t m, int n,
-                                                           float eps) {
+                                                           float eps, const float* res32, float* out32) {
   __shared__ float red[2][kBlock / kWave];
   const int64_t row = blockIdx.x;
   T* orow = out + row * n;
-  const T* irow = ADD ? input + row * n : nullptr;
+  const T* irow = (ADD && !RES32) ? input + row * n : nullptr;
+  const float* rrow = RES32 ? res32 + row * n : nullptr;
   float sum = 0.f, sumsq = 0.f;
   for (int c = threadIdx.x; c < n; c += kBlock) {
     float x = to_float(orow[c]);
-    if (ADD) x = x + to_float(irow[c]) + to_float(bias[c]);
+    if (ADD) x = x + (RES32 ? rrow[c] : to_float(irow[c])) + to_float(bias[c]);
     sum += x;
     sumsq += x * x;
   }
@@ -110,33 +122,37 @@ __global__ __launch_bounds__(kBlock) void layer_norm_block(T* __restrict__ out, 
   const float rstd = 1.0f / sqrtf(var + eps);
   for (int c = threadIdx.x; c < n; c += kBlock) {
     float x = to_float(orow[c]);
-    if (ADD) x = x + to_float(irow[c]) + to_float(bias[c]);
-    orow[c] = from_float<T>(to_float(beta[c]) + to_float(gamma[c]) * rstd * (x - mean));
+    if (ADD) x = x + (RES32 ? rrow[c] : to_float(irow[c])) + to_float(bias[c]);
+    const float y = to_float(beta[c]) + to_float(gamma[c]) * rstd * (x - mean);
+    orow[c] = from_float<T>(y);
+    if (RES32) out32[row * n + c] = y;
   }
 }
 
-template <typename T, int VEC, int G, int ITERS, bool ADD>
+template <typename T, int VEC, int G, int ITERS, bool ADD, bool RES32>
 static int launch_ln_rows(T* out, const T* input, const T* bias, const T* gamma, const T* beta, int64_t m,
-                          int n, float eps, hipStream_t s) {
+                          int n, float eps, const float* res32, float* out32, hipStream_t s) {
   constexpr int ROWS = kBlock / G;
   const int64_t grid = ceil_div(m, ROWS);
-  hipLaunchKernelGGL((layer_norm_rows<T, VEC, G, ITERS, ADD>), dim3((unsigned)grid), dim3(kBlock), 0, s, out,
-                     input, bias, gamma, beta, m, n, eps);
+  hipLaunchKernelGGL((layer_norm_rows<T, VEC, G, ITERS, ADD, RES32>), dim3((unsigned)grid), dim3(kBlock), 0, s,
+                     out, input, bias, gamma, beta, m, n, eps, res32, out32);
   return launch_status("layer_norm_rows");
 }
 
-template <typename T, bool ADD>
+template <typename T, bool ADD, bool RES32 = false>
 static int layer_norm_dispatch(T* out, const T* input, const T* bias, const T* gamma, const T* beta,
-                               int64_t m, int64_t n, float eps, hipStream_t s) {
+                               int64_t m, int64_t n, float eps, hipStream_t s, const float* res32 = nullptr,
+                               float* out32 = nullptr) {
   if (m == 0 || n == 0) return 0;
   constexpr int VEC = 16 / sizeof(T);
   auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   const bool vec_ok = (n % VEC == 0) && aligned16(out) && aligned16(gamma) && aligned16(beta) &&
-                      (!ADD || (aligned16(input) && aligned16(bias)));
+                      (!ADD || ((RES32 || aligned16(input)) && aligned16(bias)));
   if (vec_ok) {
     const int64_t nv = n / VEC;  // 16-byte vectors per row
     // Pick the group width G so that nv = G * ITERS with as little idle lane time as possible.
-#define TTMI_LN_CASE(G, ITERS) return launch_ln_rows<T, VEC, G, ITERS, ADD>(out, input, bias, gamma, beta, m, (int)n, eps, s)
+#define TTMI_LN_CASE(G, ITERS) \
+  return launch_ln_rows<T, VEC, G, ITERS, ADD, RES32>(out, input, bias, gamma, beta, m, (int)n, eps, res32, out32, s)
     if (nv <= 16) TTMI_LN_CASE(16, 1);
     if (nv <= 32) TTMI_LN_CASE(32, 1);
     if (nv <= 64) TTMI_LN_CASE(64, 1);
@@ -149,8 +165,8 @@ static int layer_norm_dispatch(T* out, const T* input, const T* bias, const T* g
 #undef TTMI_LN_CASE
   }
   TTMI_REQUIRE(m < (1ll << 31), "too many rows");
-  hipLaunchKernelGGL((layer_norm_block<T, ADD>), dim3((unsigned)m), dim3(kBlock), 0, s, out, input, bias,
-                     gamma, beta, m, (int)n, eps);
+  hipLaunchKernelGGL((layer_norm_block<T, ADD, RES32>), dim3((unsigned)m), dim3(kBlock), 0, s, out, input, bias,
+                     gamma, beta, m, (int)n, eps, res32, out32);
   return launch_status("layer_norm_block");
 }
 
@@ -345,6 +361,18 @@ int ttmi_add_bias_layer_norm(void* out, const void* input, const void* bias, con
   TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, true>((T*)out, (const T*)input, (const T*)bias,
                                                                       (const T*)gamma, (const T*)beta, m, n, eps,
                                                                       (hipStream_t)stream)));
+  return 0;
+}
+
+int ttmi_add_bias_layer_norm_residual32(void* out, const float* residual_f32, const void* bias, const void* gamma,
+                                        const void* beta, float* out_f32, int64_t m, int64_t n, float eps,
+                                        int dtype, void* stream) {
+  TTMI_REQUIRE(out && residual_f32 && bias && gamma && beta && out_f32, "null tensor");
+  TTMI_REQUIRE(m >= 0 && n >= 0 && n < (1ll << 31), "bad shape");
+  TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, true, true>((T*)out, nullptr, (const T*)bias,
+                                                                            (const T*)gamma, (const T*)beta, m, n,
+                                                                            eps, (hipStream_t)stream, residual_f32,
+                                                                            out_f32)));
   return 0;
 }
 

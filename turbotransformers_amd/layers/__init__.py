@@ -1,0 +1,14 @@
+from .modeling_bert import (BertEmbeddings, BertIntermediate, BertOutput, BertAttention, BertLayer, SequencePool,
+                            BertEncoder, BertModel, BertModelNoPooler, PoolingType, BertPooler)
+from .modeling_smart_pad import (MultiHeadedAttentionSmartBatch, BertLayerSmartBatch, BertEncoderSmartBatch,
+                                 BertModelNoPoolerSmartBatch, BertModelSmartBatch)
+from .modeling_albert import (AlbertEmbeddings, AlbertAttention, AlbertLayer, AlbertLayerGroup, AlbertTransformer,
+                              AlbertModel)
+from .return_type import ReturnType
+
+__all__ = [
+    'BertEmbeddings', 'BertIntermediate', 'BertOutput', 'BertAttention', 'BertLayer', 'BertEncoder', 'BertModel',
+    'BertModelNoPooler', 'ReturnType', 'BertPooler', 'SequencePool', 'PoolingType', 'MultiHeadedAttentionSmartBatch',
+    'BertLayerSmartBatch', 'BertEncoderSmartBatch', 'BertModelNoPoolerSmartBatch', 'BertModelSmartBatch',
+    'AlbertEmbeddings', 'AlbertAttention', 'AlbertLayer', 'AlbertLayerGroup', 'AlbertTransformer', 'AlbertModel',
+]

@@ -1,0 +1,286 @@
+#!/usr/bin/env python3
+"""Throughput / latency benchmark of the BERT encoder path on one MI355X.
+
+Protocol (the reference's: benchmark/turbo_benchmark_helper.py:29-34, benchmark_helper.py:17-61):
+a random-init HuggingFace ``BertModel(BertConfig())`` (N(0,0.02) weights, pooler included) is
+converted with ``turbo_transformers.BertModel.from_torch(model, device, "turbo")`` and run on
+uniform random ids; W untimed warm-up forwards, then K timed ones.  A "step" is one forward of
+the whole batch; sequences/s = batch / step time.
+
+Headline workload: BERT-base fp16, batch 64 x seq 512 (the shape the MFMA/HBM targets are
+stated on).  The same JSON line carries the other shapes of the metric (batch 1/20, seq 128,
+the 20-request variable-length batch), the roofline of the dominant kernel measured live with
+HIP events, and the CPU oracle timed on the host cores of the same box.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
+"""
+import argparse
+import ctypes
+import json
+import os
+import random
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3, "i8": 5000.0}
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (layers, hidden, heads, ffn, dtype, batch, seq)
+    "base_f16_b64_s512": (12, 768, 12, 3072, "f16", 64, 512),
+    "base_f16_b20_s128": (12, 768, 12, 3072, "f16", 20, 128),
+    "base_f16_b1_s128": (12, 768, 12, 3072, "f16", 1, 128),
+    "base_f32_b1_s128": (12, 768, 12, 3072, "f32", 1, 128),
+    "base_f32_b64_s512": (12, 768, 12, 3072, "f32", 64, 512),
+    "large_bf16_b64_s512": (24, 1024, 16, 4096, "bf16", 64, 512),
+}
+SMART_LENS_SEED = 0  # random.seed(0); randint(5, 500) x 20  (benchmark/benchmark_helper.py:77-79)
+
+
+def forward_flops(layers, hidden, ffn, tokens, batch, seq):
+    gemm = 2 * hidden * (3 * hidden + hidden + 2 * ffn) * tokens * layers
+    attn = 4 * seq * hidden * tokens * layers
+    return gemm, attn
+
+
+def build_model(layers, hidden, heads, ffn, dtype):
+    import torch
+    from transformers import BertConfig, BertModel
+    import turbo_transformers
+    torch.manual_seed(1234)
+    cfg = BertConfig(num_hidden_layers=layers, hidden_size=hidden, num_attention_heads=heads, intermediate_size=ffn)
+    model = BertModel(cfg).eval()
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
+    model = model.to(tdt)
+    dev = torch.device("cuda:0")
+    return turbo_transformers.BertModel.from_torch(model, dev, "turbo"), model, cfg
+
+
+def time_steps(fn, steps, warmup):
+    """-> (mean ms per step, p50 ms, list of per-step ms); events on torch's current stream, which is
+    the stream the kernels are enqueued on."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    events[0].record()
+    for i in range(steps):
+        fn()
+        events[i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = [events[i].elapsed_time(events[i + 1]) for i in range(steps)]
+    total = events[0].elapsed_time(events[steps])
+    per_sorted = sorted(per)
+    return total / steps, per_sorted[len(per) // 2], per, wall_ms / steps
+
+
+def run_dense(name, steps, warmup):
+    import torch
+    layers, hidden, heads, ffn, dtype, batch, seq = WORKLOADS[name]
+    tmodel, hf_model, cfg = build_model(layers, hidden, heads, ffn, dtype)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, cfg.vocab_size - 1, (batch, seq), generator=g, dtype=torch.int64).cuda()
+    ms, p50, _, wall = time_steps(lambda: tmodel(ids), steps, warmup)
+    gemm, attn = forward_flops(layers, hidden, ffn, batch * seq, batch, seq)
+    return {"workload": name, "dtype": dtype, "batch": batch, "seq": seq, "ms_per_step": ms, "p50_ms": p50,
+            "host_wall_ms_per_step": wall, "seq_per_s": batch / ms * 1e3,
+            "tflops": (gemm + attn) / ms / 1e9, "frac_of_mfma_peak": (gemm + attn) / ms / 1e9 / PEAK_TFLOPS[dtype]}
+
+
+def run_smart_batch(steps, warmup):
+    """20 requests with lengths from the reference's recipe, packed (no padding) vs padded to the
+    longest with a HuggingFace-style attention mask."""
+    import torch
+    import turbo_transformers
+    random.seed(SMART_LENS_SEED)
+    lens = [random.randint(5, 500) for _ in range(20)]
+    layers, hidden, heads, ffn = 12, 768, 12, 3072
+    tmodel, hf_model, cfg = build_model(layers, hidden, heads, ffn, "f16")
+    smart = turbo_transformers.BertModelSmartBatch.from_torch(hf_model, torch.device("cuda:0"))
+    g = torch.Generator().manual_seed(0)
+    inputs = [torch.randint(0, cfg.vocab_size - 1, (1, n), generator=g, dtype=torch.int64).cuda() for n in lens]
+    ms_s, p50_s, _, _ = time_steps(lambda: smart(inputs, lens), steps, warmup)
+    max_len = max(lens)
+    padded = torch.zeros(len(lens), max_len, dtype=torch.int64)
+    mask = torch.zeros(len(lens), max_len, dtype=torch.int64)
+    for i, t in enumerate(inputs):
+        padded[i, :lens[i]] = t[0].cpu()
+        mask[i, :lens[i]] = 1
+    padded, mask = padded.cuda(), mask.cuda()
+    ms_p, p50_p, _, _ = time_steps(lambda: tmodel(padded, attention_masks=mask), steps, warmup)
+    return {"workload": "base_f16_smart_batch_20req", "lens_sum": sum(lens), "lens_max": max_len,
+            "packed": {"ms_per_step": ms_s, "p50_ms": p50_s, "seq_per_s": len(lens) / ms_s * 1e3},
+            "padded": {"ms_per_step": ms_p, "p50_ms": p50_p, "seq_per_s": len(lens) / ms_p * 1e3}}
+
+
+def kernel_rooflines(dtype="f16", batch=64, seq=512, hidden=768, heads=12, ffn=3072, iters=20):
+    """Each kernel of the layer alone, at its real shape, timed with HIP events on the work stream
+    through the C ABI.  GEMMs: algorithmic FLOPs = 2*M*N*K against the MFMA peak; memory-bound
+    kernels: algorithmic bytes (each tensor read / written once) against 8 TB/s."""
+    import torch
+    from turbotransformers_amd import capi
+    lib = capi.load()
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
+    cdt = {"f16": capi.F16, "bf16": capi.BF16, "f32": capi.F32}[dtype]
+    esz = 2 if dtype != "f32" else 4
+    T, H, F, d = batch * seq, hidden, ffn, hidden // heads
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    S = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rnd = lambda *shape: (torch.randn(*shape, device="cuda") * 0.5).to(tdt)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters * 1e3  # us
+
+    x, w_qkv, w_o, w_1, w_2 = rnd(T, H), rnd(3 * H, H), rnd(H, H), rnd(F, H), rnd(H, F)
+    b_qkv, b_h, b_f, gam = rnd(3 * H), rnd(H), rnd(F), rnd(H)
+    q, k, v = (torch.empty(batch, heads, seq, d, device="cuda", dtype=tdt) for _ in range(3))
+    score = torch.empty(batch, heads, seq, seq, device="cuda", dtype=tdt)
+    ctx, out, inter = torch.empty(T, H, device="cuda", dtype=tdt), torch.empty(T, H, device="cuda", dtype=tdt), rnd(T, F)
+    mask = torch.zeros(batch, seq, device="cuda")
+
+    def fused(a, w, c, m, n, kk, epi, **kw):
+        args = capi.EpilogueArgs()
+        for key, val in kw.items():
+            setattr(args, key, val.data_ptr() if isinstance(val, torch.Tensor) else val)
+        return lambda: capi.check(lib.ttmi_gemm_fused(P(a), P(w), P(c) if c is not None else None, m, n, kk, kk, kk, n, epi,
+                                                      ctypes.byref(args), cdt, S()))
+
+    res = {}
+    gemms = {
+        "qkv_gemm+bias+split": (fused(x, w_qkv, None, T, 3 * H, H, capi.EPI_QKV_SPLIT, bias=b_qkv, q=q, k=k, v=v, seq=seq,
+                                      heads=heads, head_dim=d), 2 * T * 3 * H * H),
+        "attn_out_gemm": (lambda: capi.check(lib.ttmi_gemm(P(ctx), P(w_o), P(out), T, H, H, H, H, H, 1, 1.0, 0.0, cdt, S())),
+                          2 * T * H * H),
+        "ffn1_gemm+bias+gelu": (fused(x, w_1, inter, T, F, H, capi.EPI_BIAS_ACT, bias=b_f, act=capi.ACT_GELU), 2 * T * F * H),
+        "ffn2_gemm": (lambda: capi.check(lib.ttmi_gemm(P(inter), P(w_2), P(out), T, H, F, F, F, H, 1, 1.0, 0.0, cdt, S())),
+                      2 * T * H * F),
+        "qk_batched_gemm": (lambda: capi.check(lib.ttmi_gemm_strided_batched(
+            P(q), P(k), P(score), seq, seq, d, d, d, seq, seq * d, seq * d, seq * seq, batch * heads, 1, 0.125, 0.0, cdt, S())),
+            2 * T * seq * H),
+        "pv_batched_gemm+merge": (lambda: capi.check(lib.ttmi_gemm_batched_heads(
+            P(score), P(v), P(ctx), seq, d, seq, seq, d, H, heads, heads * seq * seq, seq * seq, heads * seq * d, seq * d,
+            seq * H, d, batch, 0, 1.0, 0.0, cdt, S())), 2 * T * seq * H),
+    }
+    for name, (fn, flops) in gemms.items():
+        us = timed(fn)
+        res[name] = {"bound": "mfma", "us": us, "achieved": flops / us / 1e6, "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
+                     "frac": flops / us / 1e6 / PEAK_TFLOPS[dtype], "flops_per_launch": flops}
+    score.normal_()
+    membound = {
+        "apply_mask_and_softmax": (lambda: capi.check(lib.ttmi_apply_mask_and_softmax(
+            P(score), P(mask), batch, heads, seq, seq, 1, 1.0, cdt, S())), 2 * batch * heads * seq * seq * esz + batch * seq * 4),
+        "add_bias_layer_norm": (lambda: capi.check(lib.ttmi_add_bias_layer_norm(
+            P(out), P(x), P(b_h), P(gam), P(b_h), T, H, 1e-12, cdt, S())), 3 * T * H * esz),
+        "add_bias_gelu": (lambda: capi.check(lib.ttmi_add_bias_act(P(inter), P(b_f), T, F, capi.ACT_GELU, cdt, S())),
+                          2 * T * F * esz),
+    }
+    for name, (fn, nbytes) in membound.items():
+        us = timed(fn)
+        res[name] = {"bound": "hbm", "us": us, "achieved": nbytes / us / 1e3, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": nbytes / us / 1e3 / PEAK_HBM_GBS, "bytes_per_launch": nbytes}
+    return res
+
+
+def cpu_baseline(seqs=4, seq=512, repeats=2):
+    """The CPU oracle (an in-repo restatement of the reference's CPU branch: OpenMP loops + cblas_sgemm)
+    on a bounded sample of the headline workload: `seqs` of the 64 sequences, all 12 layers, fp32."""
+    import numpy as np
+    from oracle.loader import Oracle
+    o = Oracle()
+    threads = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
+    o.set_num_threads(threads)
+    rng = np.random.default_rng(1234)
+    H, F, heads, L = 768, 3072, 12, 12
+    n = lambda *s: (rng.standard_normal(s, np.float32) * 0.02)
+    layers = [{"qkv_w": n(H, 3 * H), "qkv_b": np.zeros(3 * H, np.float32), "attn_out_w": n(H, H),
+               "attn_out_b": np.zeros(H, np.float32), "attn_ln_g": np.ones(H, np.float32), "attn_ln_b": np.zeros(H, np.float32),
+               "inter_w": n(H, F), "inter_b": np.zeros(F, np.float32), "out_w": n(F, H), "out_b": np.zeros(H, np.float32),
+               "out_ln_g": np.ones(H, np.float32), "out_ln_b": np.zeros(H, np.float32)} for _ in range(L)]
+    x = rng.standard_normal((seqs, seq, H), np.float32)
+    mask = np.zeros((seqs, 1, 1, seq), np.float32)
+    o.bert_encoder(x[:1, :64].copy(), mask[:1, :, :, :64].copy(), layers, heads)  # warm-up (thread pools, BLAS init)
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        o.bert_encoder(x, mask, layers, heads)
+    dt = (time.perf_counter() - t0) / repeats
+    return {"value": seqs / dt, "unit": "seq/s", "cores": threads, "kind": "port",
+            "sample": "%d of the 64 sequences (batch %d x seq %d), 12 encoder layers, fp32, %d timed forwards after a warm-up; "
+                      "BLAS: %s" % (seqs, seqs, seq, repeats, os.path.basename(o.blas_name())),
+            "seconds_per_forward": dt}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="base_f16_b64_s512", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extras", action="store_true", help="skip the other shapes of the metric")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline pass")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU (requests are independent; there is no multi-GPU step to time); "
+                 "--gpus %d is not supported" % args.gpus)
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import turbo_transformers  # noqa: F401  (fails loudly if the native libraries are missing)
+
+    head = run_dense(args.workload, args.steps, args.warmup)
+    layers, hidden, heads, ffn, dtype, batch, seq = WORKLOADS[args.workload]
+    line = {
+        "metric": "bert_base_sequences_per_second", "value": head["seq_per_s"], "unit": "seq/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "p50_latency_ms": head["p50_ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": "%s: %d-layer BERT (hidden %d, %d heads, FFN %d, pooler) %s, batch %d x seq %d, random-init "
+                               "N(0,0.02) weights, uniform random ids, via turbo_transformers.BertModel.from_torch"
+                               % (args.workload, layers, hidden, heads, ffn, dtype, batch, seq)},
+        "forward_tflops": head["tflops"], "forward_frac_of_mfma_peak": head["frac_of_mfma_peak"],
+        "device": turbo_transformers.cxx.device_info()["name"],
+    }
+    if not args.no_kernels:
+        kr = kernel_rooflines(dtype, batch, seq, hidden, heads, ffn)
+        # dominant kernel = largest share of the layer time
+        dom = max(kr, key=lambda k: kr[k]["us"])
+        r = kr[dom]
+        line["roofline"] = {"kernel": dom, "bound": r["bound"], "achieved": r["achieved"], "peak": r["peak"], "unit": r["unit"],
+                            "frac": r["frac"], "traffic": None, "avg_launch_us": r["us"]}
+        line["kernel_rooflines"] = {k: {"bound": v["bound"], "us": round(v["us"], 1), "achieved": round(v["achieved"], 1),
+                                        "unit": v["unit"], "frac": round(v["frac"], 4)} for k, v in kr.items()}
+    else:
+        line["roofline"] = None
+    if not args.no_extras:
+        extras = {}
+        for name in ("base_f16_b1_s128", "base_f16_b20_s128", "base_f32_b1_s128"):
+            if name != args.workload:
+                r = run_dense(name, max(20, args.steps), args.warmup)
+                extras[name] = {k: r[k] for k in ("ms_per_step", "p50_ms", "seq_per_s", "host_wall_ms_per_step")}
+        extras["smart_batch"] = run_smart_batch(max(10, args.steps // 2), args.warmup)
+        line["other_workloads"] = extras
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -238,6 +238,18 @@ TTMI_API int ttmi_gemm_batched_heads(const void* a, const void* b, void* c, int6
                                      int64_t c_head, int64_t batch, int trans_b, float alpha, float beta,
                                      int dtype, void* stream);
 
+/* Self-attention core in one kernel, for head_dim 64 and fp16/bf16:
+ *   out[b, s, head*64 + :] = softmax(scale * q[b,head,s,:] k[b,head]^T + mask[b,:]) v[b,head]
+ * q,k,v are [B,h,S,64]; `mask` is an additive fp32 [B,S] key mask or NULL; `out` is [B,S,h*64].
+ * It replaces BatchMatMul + ApplyMaskAndSoftmax + BatchMatMul + TransposeForScore
+ * (layers/multi_headed_attention.cpp:323-354) when the [B,h,S,S] probabilities are not an
+ * output: the score tensor never reaches HBM.  With `cu_seqlens` (device int32 [B+1]) q,k,v are
+ * the zero-padded tensors of a packed batch (S = max length): keys and queries >= len[b] are
+ * skipped and `out` is packed [sum(len), h*64] (…smart_batch.cpp:368-392). */
+TTMI_API int ttmi_fused_attention(const void* q, const void* k, const void* v, const float* mask, void* out,
+                                  const int32_t* cu_seqlens, int64_t batch, int64_t heads, int64_t seq,
+                                  int64_t head_dim, float scale, int dtype, void* stream);
+
 /* Arguments of the fused epilogues; unused members are NULL / 0. */
 typedef struct ttmi_epilogue_args {
   const void* bias;          /* [N], same dtype as C                                        */

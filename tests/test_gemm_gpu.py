@@ -229,3 +229,49 @@ def test_int8_linear_pipeline(ttmi, oracle):
     want = oracle.dequant_bias(acc_want, sx_want, sw, bias)
     assert max_abs(host(out), want) <= 1e-5
     assert max_abs(want, x @ w.T + bias) < 0.05  # and the scheme itself approximates the fp32 Linear
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("B,h,S,masked", [(2, 3, 128, True), (1, 2, 512, False), (3, 2, 100, True), (2, 1, 37, True),
+                                         (1, 1, 500, True), (2, 12, 64, False), (1, 2, 1, False), (1, 1, 700, True)])
+def test_fused_attention_vs_unfused_oracle(ttmi, oracle, dt, B, h, S, masked):
+    """One-kernel softmax(scale QK^T + mask) V against the oracle's four-step chain
+    (BatchMatMul, ApplyMaskAndSoftmax, BatchMatMul, TransposeForScore)."""
+    rng = np.random.default_rng(S + B)
+    d = 64
+    Q, K, V = (rng.standard_normal((B, h, S, d), np.float32) for _ in range(3))
+    mask = None
+    if masked:
+        mask = np.zeros((B, 1, 1, S), np.float32)
+        mask[0, ..., S // 2 + 1:] = -10000.0
+        mask[-1, ..., :S // 3] = -10000.0
+    dQ, dK, dV = dev(Q, dt), dev(K, dt), dev(V, dt)
+    out = torch.full((B, S, h * d), 9.0, dtype=dQ.dtype, device="cuda")
+    ok(ttmi.ttmi_fused_attention(ptr(dQ), ptr(dK), ptr(dV), ptr(dev(mask)) if masked else None, ptr(out), None, B, h, S, d,
+                                 0.125, TTMI_DTYPES[dt], stream()))
+    score = oracle.batch_matmul(rounded(Q, dt), rounded(K, dt), True, 0.125)
+    prob = oracle.apply_mask_and_softmax(score, mask, 1.0, True)
+    want = oracle.transpose_for_score(oracle.batch_matmul(prob, rounded(V, dt), False)).reshape(B, S, h * d)
+    # P is rounded to 16 bits before the second MFMA, as the unfused path stores it
+    assert max_abs(host(out), want) <= GEMM_TOL[dt] * 2
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+def test_fused_attention_packed_batch(ttmi, oracle, dt):
+    rng = np.random.default_rng(17)
+    lens, h, d = [70, 5, 129, 33], 2, 64
+    B, maxS, total = len(lens), max(lens), sum(lens)
+    Q, K, V = (rng.standard_normal((B, h, maxS, d), np.float32) for _ in range(3))
+    for b, L in enumerate(lens):  # pad rows are zero in the real pipeline
+        Q[b, :, L:], K[b, :, L:], V[b, :, L:] = 0, 0, 0
+    cu = np.zeros(B + 1, np.int32)
+    cu[1:] = np.cumsum(lens)
+    mask = np.where(np.arange(maxS)[None, :] < np.array(lens)[:, None], 0.0, -1e9).astype(np.float32)
+    out = torch.full((total, h * d), 9.0, dtype=dev(Q, dt).dtype, device="cuda")
+    ok(ttmi.ttmi_fused_attention(ptr(dev(Q, dt)), ptr(dev(K, dt)), ptr(dev(V, dt)), ptr(dev(mask)), ptr(out), ptr(dev(cu)), B, h,
+                                 maxS, d, 0.125, TTMI_DTYPES[dt], stream()))
+    score = oracle.batch_matmul(rounded(Q, dt), rounded(K, dt), True, 0.125)
+    prob = oracle.apply_mask_and_softmax(score, mask.reshape(B, 1, 1, maxS), 1.0, True)
+    ctx = oracle.batch_matmul(prob, rounded(V, dt), False)
+    want = oracle.transpose_for_score_pad(ctx, lens).reshape(total, h * d)
+    assert max_abs(host(out), want) <= GEMM_TOL[dt] * 2

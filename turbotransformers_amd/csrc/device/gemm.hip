@@ -114,42 +114,138 @@ struct GemmArgs {
 };
 
 // ------------------------------------------------------------------------ epilogues -----
-// Each epilogue sees (batch z, row m, column n, accumulator value) once per element; lanes
-// of a wavefront hold 32 consecutive columns of one row, so stores are 64..128-byte runs.
+// After the K loop each wavefront transposes its accumulators through LDS so that a lane holds
+// 8 consecutive columns of one row; an epilogue then sees (batch z, row m, first column n,
+// 8 accumulator values, how many of them are inside the matrix) and writes them with one
+// 16-byte store (two for fp32/int32 outputs).  `vec` (set on the host) says whether bases and
+// leading dimensions allow 16-byte accesses; otherwise, and on the ragged right edge, the
+// epilogue falls back to element stores.
+template <typename T>
+__device__ __forceinline__ void store_row8(T* p, const float (&v)[8]) {
+  if constexpr (sizeof(T) == 2) {
+    Vec<T, 8> o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o.v[j] = from_float<T>(v[j]);
+    store_vec<T, 8>(p, o);
+  } else {
+    Vec<T, 4> lo, hi;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      lo.v[j] = from_float<T>(v[j]);
+      hi.v[j] = from_float<T>(v[j + 4]);
+    }
+    store_vec<T, 4>(p, lo);
+    store_vec<T, 4>(p + 4, hi);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void load_row8(const T* p, float (&v)[8]) {
+  if constexpr (sizeof(T) == 2) {
+    Vec<T, 8> x = load_vec<T, 8>(p);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = to_float(x.v[j]);
+  } else {
+    Vec<T, 4> lo = load_vec<T, 4>(p), hi = load_vec<T, 4>(p + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = to_float(lo.v[j]);
+      v[j + 4] = to_float(hi.v[j]);
+    }
+  }
+}
+
+// Per-lane column state of an epilogue: the 8 bias values of the lane's columns.
+struct Bias8 {
+  float b[8];
+};
+
+template <typename T>
+__device__ __forceinline__ Bias8 load_bias8(const T* bias, int n, int n_limit, bool vec) {
+  Bias8 r;
+  if (bias == nullptr) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r.b[j] = 0.f;
+  } else if (vec && n + 8 <= n_limit) {
+    load_row8<T>(bias + n, r.b);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r.b[j] = (n + j < n_limit) ? to_float(bias[n + j]) : 0.f;
+  }
+  return r;
+}
+
 template <typename T>
 struct EpiAlphaBeta {
+  using Acc = float;
   T* c;
   int64_t ldc, c_outer, c_inner;
   int inner;
   float alpha, beta;
-  __device__ __forceinline__ float col(int) const { return 0.f; }
-  __device__ __forceinline__ void store(int z, int m, int n, float v, float) const {
+  bool vec;
+  __device__ __forceinline__ Bias8 prepare(int, int) const { return Bias8{}; }
+  __device__ __forceinline__ void store8(int z, int m, int n, float (&v)[8], int valid, const Bias8&) const {
     T* p = c + (int64_t)(z / inner) * c_outer + (int64_t)(z % inner) * c_inner + (int64_t)m * ldc + n;
-    float r = alpha * v;
-    if (beta != 0.f) r += beta * to_float(*p);
-    *p = from_float<T>(r);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] *= alpha;
+    if (vec && valid == 8) {
+      if (beta != 0.f) {
+        float old[8];
+        load_row8<T>(p, old);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] += beta * old[j];
+      }
+      store_row8<T>(p, v);
+    } else {
+      for (int j = 0; j < valid; ++j) {
+        float r = v[j];
+        if (beta != 0.f) r += beta * to_float(p[j]);
+        p[j] = from_float<T>(r);
+      }
+    }
   }
 };
 
 template <typename T, int ACT, bool HAS_ACT, bool HAS_RES>
 struct EpiBias {
+  using Acc = float;
   T* c;
   const T* bias;
   const T* residual;
   int64_t ldc;
-  __device__ __forceinline__ float col(int n) const { return to_float(bias[n]); }
-  __device__ __forceinline__ void store(int, int m, int n, float v, float bias_n) const {
-    float r = v + bias_n;
-    if (HAS_ACT) r = apply_act<ACT>(r);
-    if (HAS_RES) r += to_float(residual[(int64_t)m * ldc + n]);
-    c[(int64_t)m * ldc + n] = from_float<T>(r);
+  bool vec;
+  __device__ __forceinline__ Bias8 prepare(int n, int n_limit) const { return load_bias8<T>(bias, n, n_limit, vec); }
+  __device__ __forceinline__ void store8(int, int m, int n, float (&v)[8], int valid, const Bias8& bs) const {
+    const int64_t off = (int64_t)m * ldc + n;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      v[j] += bs.b[j];
+      if (HAS_ACT) v[j] = apply_act<ACT>(v[j]);
+    }
+    if (vec && valid == 8) {
+      if (HAS_RES) {
+        float res[8];
+        load_row8<T>(residual + off, res);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] += res[j];
+      }
+      store_row8<T>(c + off, v);
+    } else {
+      for (int j = 0; j < valid; ++j) {
+        float r = v[j];
+        if (HAS_RES) r += to_float(residual[off + j]);
+        c[off + j] = from_float<T>(r);
+      }
+    }
   }
 };
 
 // acc + bias -> q,k,v[B,h,S,d].  Row m is token (b,s); PAD: packed token -> padded row through
-// the per-token map token_rows[m] = b*max_seq + s.
+// the per-token map token_rows[m] = b*max_seq + s.  head_dim % 8 == 0 keeps a lane's 8 columns
+// inside one head, so they land as one 16-byte store; otherwise elements are placed one by one.
 template <typename T, bool PAD>
 struct EpiQkvSplit {
+  using Acc = float;
   T* q;
   T* k;
   T* v;
@@ -157,25 +253,51 @@ struct EpiQkvSplit {
   const int32_t* token_rows;
   int seq, heads, dim, hidden;
   FastDiv div_seq, div_hidden, div_dim;
-  __device__ __forceinline__ float col(int n) const { return to_float(bias[n]); }
-  __device__ __forceinline__ void store(int, int m, int n, float val, float bias_n) const {
-    uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;  // b*seq + s
-    const uint32_t b = div_seq.div(prow);
-    const uint32_t s = prow - b * seq;
-    const uint32_t w = div_hidden.div((uint32_t)n);
+  bool vec;
+  __device__ __forceinline__ Bias8 prepare(int n, int n_limit) const { return load_bias8<T>(bias, n, n_limit, vec); }
+  __device__ __forceinline__ T* dest(uint32_t b, uint32_t s, uint32_t n) const {
+    const uint32_t w = div_hidden.div(n);
     const uint32_t rem = n - w * hidden;
     const uint32_t head = div_dim.div(rem);
     const uint32_t i = rem - head * dim;
     T* base = (w == 0) ? q : (w == 1 ? k : v);
-    base[(((int64_t)b * heads + head) * seq + s) * dim + i] = from_float<T>(val + bias_n);
+    return base + (((int64_t)b * heads + head) * seq + s) * dim + i;
+  }
+  __device__ __forceinline__ void store8(int, int m, int n, float (&val)[8], int valid, const Bias8& bs) const {
+    const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;  // b*seq + s
+    const uint32_t b = div_seq.div(prow);
+    const uint32_t s = prow - b * seq;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) val[j] += bs.b[j];
+    if (vec && valid == 8) {
+      store_row8<T>(dest(b, s, (uint32_t)n), val);
+    } else {
+      for (int j = 0; j < valid; ++j) *dest(b, s, (uint32_t)(n + j)) = from_float<T>(val[j]);
+    }
   }
 };
 
 struct EpiInt32 {
+  using Acc = int;
   int32_t* c;
   int64_t ldc;
-  __device__ __forceinline__ int col(int) const { return 0; }
-  __device__ __forceinline__ void store(int, int m, int n, int v, int) const { c[(int64_t)m * ldc + n] = v; }
+  bool vec;
+  __device__ __forceinline__ Bias8 prepare(int, int) const { return Bias8{}; }
+  __device__ __forceinline__ void store8(int, int m, int n, int (&v)[8], int valid, const Bias8&) const {
+    int32_t* p = c + (int64_t)m * ldc + n;
+    if (vec && valid == 8) {
+      Vec<int32_t, 4> lo, hi;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        lo.v[j] = v[j];
+        hi.v[j] = v[j + 4];
+      }
+      store_vec<int32_t, 4>(p, lo);
+      store_vec<int32_t, 4>(p + 4, hi);
+    } else {
+      for (int j = 0; j < valid; ++j) p[j] = v[j];
+    }
+  }
 };
 
 // -------------------------------------------------------------------------- kernel ------
@@ -324,19 +446,39 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
     __syncthreads();
   }
 
-  // epilogue: acc[i][j][e] is C[row = 8*(e/4) + 4*lhalf + e%4][col = lrow] of its 32x32 block
+  // Epilogue.  acc[i][j][e] is C[row 8*(e/4) + 4*lhalf + e%4][col lrow] of its 32x32 block.
+  // Each wavefront stages one 32-row strip of its sub-tile at a time in its own slice of LDS
+  // (the K-loop buffers are free after the last barrier), then reads it back row-major, 8
+  // columns per lane, so that global stores are full 16-byte vectors in 128-byte row segments.
+  constexpr int W = TN * 32;             // strip width (columns)
+  constexpr int LDW = W + 4;             // padded pitch in words: rows stay 16-byte aligned
+  constexpr int LANES_PER_ROW = W / 8;   // lanes sharing one row
+  constexpr int ROWS_PER_PASS = kWave / LANES_PER_ROW;
+  static_assert(NT / kWave * 32 * LDW * 4 <= 2 * STAGE, "epilogue staging exceeds the K-loop LDS");
+  AccScalar* stage = reinterpret_cast<AccScalar*>(smem) + wave * (32 * LDW);
+  const int cg = lane % LANES_PER_ROW, rp = lane / LANES_PER_ROW;
+  const int ncol = n0 + wn0 + cg * 8;
+  const int valid = min(8, g.n - ncol);
+  const Bias8 cstate = epi.prepare(ncol, g.n);
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wn0 + j * 32 + lrow;
-    if (n >= g.n) continue;
-    const auto cstate = epi.col(n);
+  for (int i = 0; i < TM; ++i) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm0 + i * 32 + 8 * (e / 4) + 4 * lhalf + (e % 4);
-        if (m < g.m) epi.store(z, m, n, (AccScalar)acc[i][j][e], cstate);
+      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = acc[i][j][e];
+#pragma unroll
+    for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
+      const int r = p * ROWS_PER_PASS + rp;
+      const int m = m0 + wm0 + i * 32 + r;
+      AccScalar v[8];
+      const Vec<AccScalar, 4> lo = load_vec<AccScalar, 4>(stage + r * LDW + cg * 8);
+      const Vec<AccScalar, 4> hi = load_vec<AccScalar, 4>(stage + r * LDW + cg * 8 + 4);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        v[t] = lo.v[t];
+        v[t + 4] = hi.v[t];
       }
+      if (m < g.m && valid > 0) epi.store8(z, m, ncol, v, valid, cstate);
     }
   }
 }
@@ -401,8 +543,9 @@ static int gemm_alpha_beta(const void* a, const void* b, void* c, int64_t m, int
   g.lda = lda; g.ldb = ldb;
   g.inner = inner;
   g.a_outer = a_outer; g.a_inner = a_inner; g.b_outer = b_outer; g.b_inner = b_inner;
-  EpiAlphaBeta<T> epi{(T*)c, ldc, c_outer, c_inner, inner, alpha, beta};
   constexpr int KPC = 16 / sizeof(T);
+  const bool c_vec = aligned16(c) && ldc % KPC == 0 && c_outer % KPC == 0 && c_inner % KPC == 0;
+  EpiAlphaBeta<T> epi{(T*)c, ldc, c_outer, c_inner, inner, alpha, beta, c_vec};
   auto mult = [](int64_t v) { return v % KPC == 0; };
   bool aligned = aligned16(a) && aligned16(b) && mult(lda) && mult(ldb) && mult(a_outer) && mult(a_inner) &&
                  mult(b_outer) && mult(b_inner);
@@ -469,29 +612,32 @@ int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n,
   TTMI_DISPATCH_FLOAT(dtype, T, {
     constexpr int KPC = 16 / sizeof(T);
     const bool aligned = aligned16(a) && aligned16(b) && lda % KPC == 0 && ldb % KPC == 0 && k % KPC == 0;
+    const bool c_vec = aligned16(c) && ldc % KPC == 0 && aligned16(args->bias) && aligned16(args->residual);
+    const bool qkv_vec = aligned16(args->q) && aligned16(args->k) && aligned16(args->v) && aligned16(args->bias) &&
+                         args->head_dim % 8 == 0;
     switch (epilogue) {
       case TTMI_EPI_BIAS: {
         TTMI_REQUIRE(c && args->bias && ldc >= n, "BIAS epilogue needs c and bias");
-        EpiBias<T, 0, false, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc};
+        EpiBias<T, 0, false, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc, c_vec};
         return (launch_gemm<T, false>(g, epi, 1, aligned, s));
       }
       case TTMI_EPI_BIAS_ACT: {
         TTMI_REQUIRE(c && args->bias && ldc >= n, "BIAS_ACT epilogue needs c and bias");
         if (args->act == TTMI_ACT_GELU) {
-          EpiBias<T, TTMI_ACT_GELU, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc};
+          EpiBias<T, TTMI_ACT_GELU, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc, c_vec};
           return (launch_gemm<T, false>(g, epi, 1, aligned, s));
         } else if (args->act == TTMI_ACT_TANH) {
-          EpiBias<T, TTMI_ACT_TANH, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc};
+          EpiBias<T, TTMI_ACT_TANH, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc, c_vec};
           return (launch_gemm<T, false>(g, epi, 1, aligned, s));
         } else if (args->act == TTMI_ACT_RELU) {
-          EpiBias<T, TTMI_ACT_RELU, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc};
+          EpiBias<T, TTMI_ACT_RELU, true, false> epi{(T*)c, (const T*)args->bias, nullptr, ldc, c_vec};
           return (launch_gemm<T, false>(g, epi, 1, aligned, s));
         }
         return fail(TTMI_EINVAL, "unknown activation");
       }
       case TTMI_EPI_BIAS_RESIDUAL: {
         TTMI_REQUIRE(c && args->bias && args->residual && ldc >= n, "BIAS_RESIDUAL epilogue needs c, bias, residual");
-        EpiBias<T, 0, false, true> epi{(T*)c, (const T*)args->bias, (const T*)args->residual, ldc};
+        EpiBias<T, 0, false, true> epi{(T*)c, (const T*)args->bias, (const T*)args->residual, ldc, c_vec};
         return (launch_gemm<T, false>(g, epi, 1, aligned, s));
       }
       case TTMI_EPI_QKV_SPLIT:
@@ -506,12 +652,12 @@ int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n,
         if (pad) {
           EpiQkvSplit<T, true> epi{(T*)args->q, (T*)args->k, (T*)args->v, (const T*)args->bias, args->token_rows,
                                    (int)args->seq, (int)args->heads, (int)args->head_dim, hidden,
-                                   FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim)};
+                                   FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim), qkv_vec};
           return (launch_gemm<T, false>(g, epi, 1, aligned, s));
         }
         EpiQkvSplit<T, false> epi{(T*)args->q, (T*)args->k, (T*)args->v, (const T*)args->bias, nullptr,
                                   (int)args->seq, (int)args->heads, (int)args->head_dim, hidden,
-                                  FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim)};
+                                  FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim), qkv_vec};
         return (launch_gemm<T, false>(g, epi, 1, aligned, s));
       }
       default:
@@ -532,7 +678,7 @@ int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_
   g.m = (int)m; g.n = (int)n; g.k = (int)k;
   g.lda = lda; g.ldb = ldb;
   g.inner = 1;
-  EpiInt32 epi{c, ldc};
+  EpiInt32 epi{c, ldc, aligned16(c) && ldc % 4 == 0};
   const bool aligned = aligned16(a) && aligned16(b) && lda % 16 == 0 && ldb % 16 == 0 && k % 16 == 0;
   return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
 }

@@ -45,15 +45,35 @@ void MultiHeadedAttention::SelfAttentionTail(const Tensor& query_tensor, const T
   const int64_t hidden = query_tensor.shape(-1), heads = num_attention_heads_, d = hidden / heads;
   const int64_t tokens = query_tensor.numel() / hidden;
 
+  ctx_.ReshapeAs(query_tensor.dtype(), {tokens, hidden}, dev, dev_id, "batch_gemm4/Reshape");
+  const float scaler = 1.0f / std::sqrt(static_cast<float>(d));
+
+  // Nobody asked for the probabilities: run the whole core as one kernel; the [B,h,S,S] scores
+  // never reach HBM.  (fp16/bf16, head size 64, key mask broadcast over query rows.)
+  bool mask_is_key_mask = true;
+  if (!attention_mask.is_null()) {
+    mask_is_key_mask = attention_mask.n_dim() == 2 || (attention_mask.n_dim() == 3 && attention_mask.shape(1) == 1) ||
+                       (attention_mask.n_dim() == 4 && attention_mask.shape(2) == 1);
+  }
+  const bool fused_core = att_score == nullptr && d == 64 && (dt == TTMI_F16 || dt == TTMI_BF16) && mask_is_key_mask;
+  if (fused_core) {
+    const float* mask = nullptr;
+    if (!attention_mask.is_null()) {
+      TT_ENFORCE_EQ(attention_mask.numel(), batch * seq, "attention mask has the wrong size");
+      mask = attention_mask.data<float>();
+    }
+    const int32_t* cu = nullptr;
+    if (seq_list != nullptr) cu = DeviceContext::GetInstance().GetSeqPlan(*seq_list).cu_seqlens;
+    TT_DEVICE_CALL(ttmi_fused_attention(q_.raw(), k_.raw(), v_.raw(), mask, ctx_.mutable_raw(), cu, batch, heads, seq, d,
+                                        scaler, dt, Stream()));
+  } else {
   Tensor* score = att_score != nullptr ? att_score : &score_scratch_;
   score->ReshapeAs(query_tensor.dtype(), {batch, heads, seq, seq}, dev, dev_id, "batch_gemm3/Reshape");
-  const float scaler = 1.0f / std::sqrt(static_cast<float>(d));
   // batch_gemm3: score[b,h] = scaler * q[b,h] k[b,h]^T   (multi_headed_attention.cpp:328-330)
   TT_DEVICE_CALL(ttmi_gemm_strided_batched(q_.raw(), k_.raw(), score->mutable_raw(), seq, seq, d, d, d, seq, seq * d,
                                            seq * d, seq * seq, batch * heads, 1, scaler, 0.f, dt, Stream()));
   kernels::ApplyMaskAndSoftmax(score, attention_mask, 1.0f);
 
-  ctx_.ReshapeAs(query_tensor.dtype(), {tokens, hidden}, dev, dev_id, "batch_gemm4/Reshape");
   if (seq_list == nullptr) {
     // batch_gemm4 with the [B,h,S,d] -> [B,S,h,d] transpose folded into the store (:345-354)
     TT_DEVICE_CALL(ttmi_gemm_batched_heads(score->raw(), v_.raw(), ctx_.mutable_raw(), seq, d, seq, seq, d, hidden, heads,
@@ -67,6 +87,7 @@ void MultiHeadedAttention::SelfAttentionTail(const Tensor& query_tensor, const T
                                              seq * d, seq * d, batch * heads, 0, 1.f, 0.f, dt, Stream()));
     kernels::TransposeForScorePad(&ctx_, padded, *seq_list);
   }
+  }  // unfused core
 
   output->ReshapeAs(query_tensor.dtype(), {query_tensor.shape(0), query_tensor.shape(1), hidden}, dev, dev_id, "gemm5/Reshape");
   const void* wo = dense_packed_.Get(dense_weight_, is_trans_weight);

@@ -35,7 +35,9 @@ class MultiHeadedAttentionSmartBatch(cxx.MultiHeadedAttentionSmartBatch):
                  layer_cache: Optional[dict] = None, attn_type: str = None, pre_layernorm: bool = False,
                  post_layernorm: bool = False, post_add_input: bool = False, is_trans_weight: bool = False,
                  return_type: Optional[ReturnType] = None, output: Optional[cxx.Tensor] = None,
-                 attn: Optional[cxx.Tensor] = None):
+                 attn: Optional[cxx.Tensor] = None, need_attn: bool = True):
+        """-> (output, attn).  need_attn=False (not in the reference signature) skips materialising
+        the padded [B,h,max_len,max_len] probabilities and returns None for them."""
         use_current_stream()
         if layer_cache:
             raise NotImplementedError("layer_cache belongs to the decoder path and is not built")
@@ -44,11 +46,12 @@ class MultiHeadedAttentionSmartBatch(cxx.MultiHeadedAttentionSmartBatch):
         if mask is None:
             mask = smart_pad_mask(query_seq_len_list if attn_type == "self" else key_seq_len_list)
         output = create_empty_if_none(output)
-        attn = create_empty_if_none(attn)
+        attn = create_empty_if_none(attn) if need_attn else None
         super().__call__(try_convert(key_tensor), try_convert(value_tensor), try_convert(query_tensor),
                          try_convert(mask), attn_type, output, attn, {}, query_seq_len_list, key_seq_len_list,
                          pre_layernorm, post_layernorm, post_add_input, is_trans_weight)
-        return convert_returns_as_type(output, return_type), convert_returns_as_type(attn, return_type)
+        return (convert_returns_as_type(output, return_type),
+                convert_returns_as_type(attn, return_type) if need_attn else None)
 
     @staticmethod
     def from_torch(attention, layer_norm=None, is_trans_weight: bool = False):
@@ -79,7 +82,8 @@ class BertLayerSmartBatch:
                  output_attentions=False, return_type: Optional[ReturnType] = None):
         attention_output, attn = self.attention(hidden_states, hidden_states, hidden_states, query_seq_len_list,
                                                 query_seq_len_list, mask=attention_mask, attn_type="self",
-                                                post_layernorm=True, return_type=ReturnType.turbo_transformers)
+                                                post_layernorm=True, return_type=ReturnType.turbo_transformers,
+                                                need_attn=bool(output_attentions))
         intermediate_output = self.intermediate(attention_output, return_type=ReturnType.turbo_transformers)
         layer_output = self.output(intermediate_output, attention_output, return_type=return_type)
         return (layer_output, attn) if output_attentions else (layer_output, )

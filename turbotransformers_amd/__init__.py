@@ -13,7 +13,7 @@ _here = _os.path.dirname(_os.path.abspath(__file__))
 try:
     from . import turbo_transformers_cxx as cxx
 except ImportError as _e:  # fail loudly: nothing works without the native module
-    raise ImportError("turbo_transformers_cxx is not built (%s); run `python -m turbotransformers_amd.build`" % _e)
+    raise ImportError("turbo_transformers_cxx is not built (%s); run `python turbotransformers_amd/build.py`" % _e)
 
 from .layers import *  # noqa: E402,F401,F403
 from .layers import __all__ as _layers_all  # noqa: E402

@@ -3,7 +3,7 @@
   libttmi.so                 HIP kernels + C ABI (hipcc, gfx950 only)
   turbo_transformers_cxx.so  host C++ layers + pybind11 module (g++), links libttmi.so
 
-Run as ``python -m turbotransformers_amd.build [device|host|all]``.  Outputs land next to
+Run as ``python turbotransformers_amd/build.py [device|host|all]``.  Outputs land next to
 the package so that they travel with the source tree; nothing is installed.
 """
 import os

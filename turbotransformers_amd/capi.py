@@ -71,7 +71,7 @@ def load(path=LIB_PATH):
     if _lib is not None:
         return _lib
     if not os.path.exists(path):
-        raise RuntimeError("libttmi.so not built (%s); run `python -m turbotransformers_amd.build`" % path)
+        raise RuntimeError("libttmi.so not built (%s); run `python turbotransformers_amd/build.py`" % path)
     lib = ctypes.CDLL(path)
     for name, (restype, argtypes) in parse_header().items():
         fn = getattr(lib, name)  # AttributeError if a declared symbol is not exported

@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void fused_attention_kernel(const T* __restric
       const int key = c >> 3, ch = c & 7;
       Chunk16 x{{0u, 0u, 0u, 0u}};
       if (key0 + key < kv_len) x = *reinterpret_cast<const Chunk16*>(kb + (int64_t)(key0 + key) * kD + ch * 8);
-      *reinterpret_cast<Chunk16*>(k_lds(stage) + key * 128 + ((ch ^ (key & 7)) << 4)) = x;
+      *reinterpret_cast<Chunk16*>(k_lds(stage) + key * 128 + ((ch ^ ((key >> 1) & 7)) << 4)) = x;
     }
     // V: thread -> (key tid&63, d-chunk (tid>>6) + 4i); scattered into V^T[d][key] so that lanes
     // write consecutive halfs of one row (no bank conflicts)
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(256) void fused_attention_kernel(const T* __restric
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
           const int key = sk + lrow;
-          const Chunk16 kf = *reinterpret_cast<const Chunk16*>(k_lds(stage) + key * 128 + (((2 * kk + lhalf) ^ (key & 7)) << 4));
+          const Chunk16 kf = *reinterpret_cast<const Chunk16*>(k_lds(stage) + key * 128 + (((2 * kk + lhalf) ^ ((key >> 1) & 7)) << 4));
           st = mma16<T>(kf, qf[kk], st);
         }
         // st[e] = score of (key sk + 8*(e/4) + 4*lhalf + e%4, query lrow)

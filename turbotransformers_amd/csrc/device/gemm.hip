@@ -301,7 +301,57 @@ struct EpiInt32 {
 };
 
 // -------------------------------------------------------------------------- kernel ------
-__device__ __forceinline__ int swizzle(int row, int chunk) { return chunk ^ (row & 7); }
+// LDS rows are 128 bytes and the LDS has 64 four-byte banks (256 bytes per bank cycle): rows r and
+// r+2 start on the same bank.  A 128-bit operand read is served 16 lanes (= 16 consecutive tile
+// rows, one chunk each) at a time, so the 16 rows must land in 16 different 16-byte slots of the
+// 256-byte bank period: slot = (r&1)*8 + physical chunk, with physical chunk = chunk ^ ((r>>1)&7).
+__device__ __forceinline__ int swizzle(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+
+// Epilogue shared by the kernels.  acc[i][j][e] is C[row 8*(e/4) + 4*lhalf + e%4][col lrow] of its
+// 32x32 block.  Each wavefront stages one 32-row strip of its sub-tile at a time in its own
+// slice of LDS (the K-loop buffers are free after the last barrier), then reads it back
+// row-major, 8 columns per lane, so that global stores are full 16-byte vectors in 128-byte
+// row segments.
+template <typename T, int TM, int TN, int NT, int LDS_BYTES, typename Epi>
+__device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], char* smem, const Epi& epi,
+                                           const GemmArgs& g, int z, int wave_m0, int wave_n0, int lane, int wave) {
+  using AccScalar = typename Mma<T>::AccScalar;
+  constexpr int W = TN * 32;             // strip width (columns)
+  constexpr int LDW = W + 4;             // padded pitch in words: rows stay 16-byte aligned
+  constexpr int LANES_PER_ROW = W / 8;   // lanes sharing one row
+  constexpr int PASSES = (32 * LANES_PER_ROW + kWave - 1) / kWave;
+  static_assert(NT / kWave * 32 * LDW * 4 <= LDS_BYTES, "epilogue staging exceeds the K-loop LDS");
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  AccScalar* stage = reinterpret_cast<AccScalar*>(smem) + wave * (32 * LDW);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = acc[i][j][e];
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int idx = p * kWave + lane;          // (row, column group) handled by this lane
+      const int r = idx / LANES_PER_ROW, cg = idx % LANES_PER_ROW;
+      if (r >= 32) continue;
+      const int m = wave_m0 + i * 32 + r;
+      const int ncol = wave_n0 + cg * 8;
+      const int valid = min(8, g.n - ncol);
+      AccScalar v[8];
+      const Vec<AccScalar, 4> lo = load_vec<AccScalar, 4>(stage + r * LDW + cg * 8);
+      const Vec<AccScalar, 4> hi = load_vec<AccScalar, 4>(stage + r * LDW + cg * 8 + 4);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        v[t] = lo.v[t];
+        v[t + 4] = hi.v[t];
+      }
+      if (m < g.m && valid > 0) {
+        const Bias8 cstate = epi.prepare(ncol, g.n);
+        epi.store8(z, m, ncol, v, valid, cstate);
+      }
+    }
+  }
+}
 
 template <typename T, int BM, int BN, int WM, int WN, bool B_KN, bool ALIGNED, typename Epi>
 __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g, const Epi epi) {
@@ -446,41 +496,165 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
     __syncthreads();
   }
 
-  // Epilogue.  acc[i][j][e] is C[row 8*(e/4) + 4*lhalf + e%4][col lrow] of its 32x32 block.
-  // Each wavefront stages one 32-row strip of its sub-tile at a time in its own slice of LDS
-  // (the K-loop buffers are free after the last barrier), then reads it back row-major, 8
-  // columns per lane, so that global stores are full 16-byte vectors in 128-byte row segments.
-  constexpr int W = TN * 32;             // strip width (columns)
-  constexpr int LDW = W + 4;             // padded pitch in words: rows stay 16-byte aligned
-  constexpr int LANES_PER_ROW = W / 8;   // lanes sharing one row
-  constexpr int ROWS_PER_PASS = kWave / LANES_PER_ROW;
-  static_assert(NT / kWave * 32 * LDW * 4 <= 2 * STAGE, "epilogue staging exceeds the K-loop LDS");
-  AccScalar* stage = reinterpret_cast<AccScalar*>(smem) + wave * (32 * LDW);
-  const int cg = lane % LANES_PER_ROW, rp = lane / LANES_PER_ROW;
-  const int ncol = n0 + wn0 + cg * 8;
-  const int valid = min(8, g.n - ncol);
-  const Bias8 cstate = epi.prepare(ncol, g.n);
+  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, smem, epi, g, z, m0 + wm0, n0 + wn0, lane, wave);
+}
+
+// ------------------------------------------------------------------ fast-path kernel -----
+// Same tiling, for the shapes the encoder actually runs (B given as [N,K], 16-byte aligned
+// operands, K a multiple of the 128-byte K step).  Two differences from the general kernel:
+//   * global -> LDS copies are `global_load_lds_dwordx4` DMA loads: a wavefront instruction
+//     moves 8 tile rows (64 lanes x 16 bytes) straight into LDS, no VGPR staging, no
+//     ds_write.  The LDS side is linear in the lane id, so the XOR swizzle is applied on the
+//     global side: lane l fills physical chunk l%8 of row l/8 and therefore fetches logical
+//     chunk (l%8) ^ ((row>>1)&7) of that row.  Rows past the M / N edge are clamped to the
+//     last valid row (their results are never stored).
+//   * MFMA operand fragments are double-buffered in registers: the LDS reads of k-substep
+//     kk+1 are issued before the MFMAs of kk.
+template <typename T, int BM, int BN, int WM, int WN, typename Epi>
+__global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmArgs g, const Epi epi) {
+  constexpr int NW = WM * WN, NT = NW * kWave;
+  constexpr int KPC = 16 / sizeof(T);
+  constexpr int BK = kRowBytes / sizeof(T);
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_LOADS = BM / 8 / NW, B_LOADS = BN / 8 / NW;  // DMA instructions per wave and K step
+  static_assert(BM / 8 % NW == 0 && BN / 8 % NW == 0, "tile rows must split evenly over the wavefronts");
+  using Acc = typename Mma<T>::Acc;
+  typedef __attribute__((address_space(3))) char lds_char;
+
+  extern __shared__ __align__(16) char smem[];
+
+  const int tiles = g.tiles_m * g.tiles_n;
+  const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
+  const int logical = (int)(blockIdx.x % kNumXcd) * per_xcd + (int)(blockIdx.x / kNumXcd);
+  if (logical >= tiles) return;
+  const int tile_m = logical / g.tiles_n, tile_n = logical % g.tiles_n;
+  const int z = blockIdx.z;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const T* A = reinterpret_cast<const T*>(g.a) + (int64_t)(z / g.inner) * g.a_outer + (int64_t)(z % g.inner) * g.a_inner;
+  const T* B = reinterpret_cast<const T*>(g.b) + (int64_t)(z / g.inner) * g.b_outer + (int64_t)(z % g.inner) * g.b_inner;
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave, wave = tid / kWave;
+  const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
+  const int lrow = lane & 31, lhalf = lane >> 5;
+
+  // per-lane source pointers of the DMA loads (advanced by one K step per iteration)
+  const T* pa[A_LOADS];
+  const T* pb[B_LOADS];
+  {
+    const int sub = lane >> 3, p = lane & 7;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int row = (wave * A_LOADS + i) * 8 + sub;
+      const int c = p ^ ((row >> 1) & 7);
+      pa[i] = A + (int64_t)min(m0 + row, g.m - 1) * g.lda + c * KPC;
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const int row = (wave * B_LOADS + i) * 8 + sub;
+      const int c = p ^ ((row >> 1) & 7);
+      pb[i] = B + (int64_t)min(n0 + row, g.n - 1) * g.ldb + c * KPC;
+    }
+  }
+  lds_char* lds0 = reinterpret_cast<lds_char*>(reinterpret_cast<uintptr_t>(smem));
+
+  // The DMA builtin exists only in the device pass; the host pass of this translation unit
+  // needs the kernel body just to emit the launch stub.
+#if defined(__HIP_DEVICE_COMPILE__)
+  auto issue = [&](int stage) {
+    lds_char* as = lds0 + stage * STAGE + wave * (A_LOADS * 1024);
+    lds_char* bs = lds0 + stage * STAGE + A_BYTES + wave * (B_LOADS * 1024);
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      __builtin_amdgcn_global_load_lds(pa[i], as + i * 1024, 16, 0, 0);
+      pa[i] += BK;
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      __builtin_amdgcn_global_load_lds(pb[i], bs + i * 1024, 16, 0, 0);
+      pb[i] += BK;
+    }
+  };
+#else
+  auto issue = [&](int) { (void)lds0; };
+#endif
+
+  Acc acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = acc[i][j][e];
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  // byte offsets of this lane's operand rows inside a stage (swizzle folded in per k-substep)
+  const int a_row0 = (wm0 + lrow) * kRowBytes, b_row0 = A_BYTES + (wn0 + lrow) * kRowBytes;
+  const int swz = ((lrow >> 1) & 7);  // rows wm0 + 32 i + lrow share (row>>1)&7 with lrow
+
+  auto read_frags = [&](const char* st, int kk, Chunk (&fa)[TM], Chunk (&fb)[TN]) {
+    const int off = ((2 * kk + lhalf) ^ swz) << 4;
 #pragma unroll
-    for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
-      const int r = p * ROWS_PER_PASS + rp;
-      const int m = m0 + wm0 + i * 32 + r;
-      AccScalar v[8];
-      const Vec<AccScalar, 4> lo = load_vec<AccScalar, 4>(stage + r * LDW + cg * 8);
-      const Vec<AccScalar, 4> hi = load_vec<AccScalar, 4>(stage + r * LDW + cg * 8 + 4);
+    for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const Chunk*>(st + a_row0 + i * 32 * kRowBytes + off);
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        v[t] = lo.v[t];
-        v[t + 4] = hi.v[t];
-      }
-      if (m < g.m && valid > 0) epi.store8(z, m, ncol, v, valid, cstate);
+    for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const Chunk*>(st + b_row0 + j * 32 * kRowBytes + off);
+  };
+
+  // Software pipeline of one K step (4 k-substeps kk, TM*TN MFMAs each):
+  //   kk = 0,1,2 : LDS reads of substep kk+1 interleaved with the MFMAs of kk
+  //   wait for the DMA of the next stage + barrier   (everyone has also read all of this stage)
+  //   issue the DMA of step kt+2 into the stage just drained
+  //   kk = 3     : LDS reads of substep 0 of the NEXT stage interleaved with the MFMAs of kk = 3
+  // so neither the LDS latency nor the barrier leaves the MFMA pipe without queued work.
+  // sched_group_barrier pins the interleaving (mask 0x100 = LDS read, 0x008 = MFMA).
+  constexpr int READS = TM + TN, MMAS = TM * TN;
+  auto mma_step = [&](Chunk (&fa)[TM], Chunk (&fb)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) Mma<T>::run(fa[i], fb[j], acc[i][j]);
+  };
+  auto interleave = [&]() {
+    // MFMA first: its operands were read one substep ago, so the wait in front of it does not
+    // cover the reads issued after it.
+    constexpr int MF = (sizeof(T) == 4) ? 4 * MMAS : MMAS;  // fp32: 4 MFMA instructions per Mma::run
+    constexpr int PER = (MF - 1) / READS;
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+    for (int r = 0; r < READS; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x008, MF - 1 - PER * READS, 0);
+  };
+
+  const int ksteps = g.k / BK;
+  issue(0);
+  __syncthreads();
+  if (ksteps > 1) issue(1);
+  Chunk fa[2][TM], fb[2][TN];
+  read_frags(smem, 0, fa[0], fb[0]);
+  for (int kt = 0; kt < ksteps; ++kt) {
+    const int cur = kt & 1;
+    const char* st = smem + cur * STAGE;
+    const char* st_next = smem + (cur ^ 1) * STAGE;
+    read_frags(st, 1, fa[1], fb[1]);
+    mma_step(fa[0], fb[0]);
+    interleave();
+    read_frags(st, 2, fa[0], fb[0]);
+    mma_step(fa[1], fb[1]);
+    interleave();
+    read_frags(st, 3, fa[1], fb[1]);
+    mma_step(fa[0], fb[0]);
+    interleave();
+    __syncthreads();
+    if (kt + 2 < ksteps) issue(cur);
+    read_frags(st_next, 0, fa[0], fb[0]);  // harmless on the last step
+    mma_step(fa[1], fb[1]);
+    interleave();
   }
+  __syncthreads();  // all LDS reads done before the epilogue reuses the buffers
+  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, smem, epi, g, z, m0 + wm0, n0 + wn0, lane, wave);
 }
 
 // ------------------------------------------------------------------------ launching -----
@@ -507,16 +681,80 @@ static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// Tile choice: the largest tile that still gives every CU work.  256x256 needs >= ~1 wave of
-// workgroups over 256 CUs to pay off; small problems (B=1, S=128) take 64x64 tiles.
+template <typename T, int BM, int BN, int WM, int WN, typename Epi>
+static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
+  constexpr int NT = WM * WN * kWave;
+  constexpr int LDS = 2 * (BM + BN) * kRowBytes;
+  g.tiles_m = (g.m + BM - 1) / BM;
+  g.tiles_n = (g.n + BN - 1) / BN;
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  TTMI_REQUIRE(tiles < (1ll << 30) && batch < 65536, "GEMM grid too large");
+  const unsigned grid_x = (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd);
+  auto kern = gemm_fast_kernel<T, BM, BN, WM, WN, Epi>;
+  if (LDS > 64 * 1024) {
+    static bool attr_set = false;  // per instantiation
+    if (!attr_set) {
+      TTMI_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+      attr_set = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3(grid_x, 1, (unsigned)batch), dim3(NT), LDS, s, g, epi);
+  return launch_status("gemm_fast_kernel");
+}
+
+// Tile configurations of the fast path and a cost model to pick one.  With t = tile area /
+// efficiency as the time of one tile on an otherwise idle CU, and `per_cu` workgroups of that
+// size resident per CU (they then share its MFMA pipes):
+//   time ~ full_rounds * per_cu * t  +  ceil(remaining_tiles / CUs) * t
+// Large tiles reuse LDS operands best (efficiency 1.0 for 256x256) but quantise badly when the
+// tile count is a small non-multiple of the 256 CUs, e.g. N = 768 at M = 32768: 384 tiles of
+// 256x256 are 1.5 rounds, 512 tiles of 256x192 are exactly 2.  Problems with few tiles take
+// the smallest tile: they are latency-bound and want as many CUs as possible.
+struct TileConfig {
+  int bm, bn, per_cu;
+  float eff;
+};
+constexpr TileConfig kTileConfigs[] = {
+    {256, 256, 1, 1.00f}, {256, 192, 1, 0.93f}, {256, 128, 1, 0.82f}, {128, 128, 2, 0.62f}, {64, 64, 4, 0.30f}};
+constexpr int kNumCus = 256;
+
+static int pick_tile(int64_t m, int64_t n, int64_t batch) {
+  int best = 0;
+  double best_cost = 1e300;
+  for (int i = 0; i < (int)(sizeof(kTileConfigs) / sizeof(kTileConfigs[0])); ++i) {
+    const TileConfig& c = kTileConfigs[i];
+    const int64_t tiles = ceil_div(m, c.bm) * ceil_div(n, c.bn) * batch;
+    const int64_t slots = (int64_t)kNumCus * c.per_cu;
+    const int64_t full = tiles / slots, rem = tiles % slots;
+    const double t = (double)c.bm * c.bn / c.eff;
+    const double cost = (double)full * c.per_cu * t + (double)ceil_div(rem, kNumCus) * t;
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = i;
+    }
+  }
+  return best;
+}
+
 template <typename T, bool B_KN, typename Epi>
 static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipStream_t s) {
   if (g.m <= 0 || g.n <= 0 || batch <= 0) return 0;
   TTMI_REQUIRE(g.k > 0, "K must be positive");
   auto tiles = [&](int bm, int bn) { return (int64_t)ceil_div(g.m, bm) * ceil_div(g.n, bn) * batch; };
   if (!B_KN) {
+    constexpr int BK = kRowBytes / sizeof(T);
+    if (aligned && g.k % BK == 0) {
+      switch (pick_tile(g.m, g.n, batch)) {
+        case 0: return launch_fast<T, 256, 256, 2, 4, Epi>(g, epi, batch, s);
+        case 1: return launch_fast<T, 256, 192, 4, 2, Epi>(g, epi, batch, s);
+        case 2: return launch_fast<T, 256, 128, 4, 2, Epi>(g, epi, batch, s);
+        case 3: return launch_fast<T, 128, 128, 2, 2, Epi>(g, epi, batch, s);
+        // small problems are latency-bound: the register-staged kernel hides the global latency
+        // of a one-step prefetch better than the DMA path does with a tiny tile
+        default: return launch_config<T, 64, 64, 2, 2, false, true, Epi>(g, epi, batch, s);
+      }
+    }
     if (aligned) {
-      if (tiles(256, 256) >= 200 && g.n >= 192 && g.m >= 192) return launch_config<T, 256, 256, 2, 4, false, true, Epi>(g, epi, batch, s);
       if (tiles(128, 128) >= 200) return launch_config<T, 128, 128, 2, 2, false, true, Epi>(g, epi, batch, s);
       return launch_config<T, 64, 64, 2, 2, false, true, Epi>(g, epi, batch, s);
     }

@@ -172,62 +172,85 @@ static int layer_norm_dispatch(T* out, const T* input, const T* bias, const T* g
 
 // ----------------------------------------------------------------------------- softmax --
 // x = score*scale + mask; p = exp(x - max) * (1/sum)        (softmax.cpp:28-81)
-template <typename T, int VEC, int G, int ITERS>
+// A group of G lanes owns R consecutive rows; all R*ITERS vector loads of score (and mask) are
+// issued before the first reduction so that enough bytes are in flight per wavefront.
+template <typename T, int VEC, int G, int ITERS, int R, bool MASK_VEC>
 __global__ __launch_bounds__(kBlock) void softmax_rows(T* __restrict__ score, const float* __restrict__ mask,
                                                        int64_t rows, int heads, int from_len, int to_len,
                                                        int mask_is_2d, float scale) {
-  constexpr int ROWS = kBlock / G;
+  constexpr int GROUPS = kBlock / G;
+  constexpr float kLowest = -3.402823466e+38f;
   const int lane = threadIdx.x % G;
-  const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / G;
-  const bool row_ok = row < rows;
-  T* srow = score + row * to_len;
-  const float* mrow = nullptr;
-  if (mask != nullptr && row_ok) {
-    const int64_t b = row / ((int64_t)heads * from_len);
-    const int64_t f = row % from_len;
-    mrow = mask + (mask_is_2d ? b * to_len : (b * from_len + f) * to_len);
-  }
-  float x[ITERS][VEC];
-  float mx = -3.402823466e+38f;
+  const int64_t row0 = ((int64_t)blockIdx.x * GROUPS + threadIdx.x / G) * R;
+  float x[R][ITERS][VEC];
 #pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int col = (it * G + lane) * VEC;
-    if (row_ok && col < to_len) {
-      Vec<T, VEC> s = load_vec<T, VEC>(srow + col);
+  for (int r = 0; r < R; ++r) {
+    const int64_t row = row0 + r;
+    const bool row_ok = row < rows;
+    const T* srow = score + row * to_len;
+    const float* mrow = nullptr;
+    if (mask != nullptr && row_ok) {
+      const int64_t b = row / ((int64_t)heads * from_len);
+      const int64_t f = row % from_len;
+      mrow = mask + (mask_is_2d ? b * to_len : (b * from_len + f) * to_len);
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int col = (it * G + lane) * VEC;
+      if (row_ok && col < to_len) {
+        const Vec<T, VEC> sv = load_vec<T, VEC>(srow + col);
+        if (mrow != nullptr) {
+          if (MASK_VEC) {
+            const Vec<float, VEC> mv = load_vec<float, VEC>(mrow + col);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) x[r][it][j] = to_float(sv.v[j]) * scale + mv.v[j];
+          } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) x[r][it][j] = to_float(sv.v[j]) * scale + mrow[col + j];
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) x[r][it][j] = to_float(sv.v[j]) * scale;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[r][it][j] = kLowest;
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t row = row0 + r;
+    const bool row_ok = row < rows;
+    float mx = kLowest;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) mx = fmaxf(mx, x[r][it][j]);
+    mx = group_max<G>(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int col = (it * G + lane) * VEC;
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        float v = to_float(s.v[j]) * scale;
-        if (mrow) v += mrow[col + j];
-        x[it][j] = v;
-        mx = fmaxf(mx, v);
+        const float e = (row_ok && col < to_len) ? __expf(x[r][it][j] - mx) : 0.f;
+        x[r][it][j] = e;
+        sum += e;
       }
-    } else {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) x[it][j] = -3.402823466e+38f;
     }
-  }
-  mx = group_max<G>(mx);
-  float sum = 0.f;
+    sum = group_sum<G>(sum);
+    const float coef = 1.0f / sum;
+    T* srow = score + row * to_len;
 #pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int col = (it * G + lane) * VEC;
+    for (int it = 0; it < ITERS; ++it) {
+      const int col = (it * G + lane) * VEC;
+      if (row_ok && col < to_len) {
+        Vec<T, VEC> o;
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      const float e = (row_ok && col < to_len) ? __expf(x[it][j] - mx) : 0.f;
-      x[it][j] = e;
-      sum += e;
-    }
-  }
-  sum = group_sum<G>(sum);
-  const float coef = 1.0f / sum;
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int col = (it * G + lane) * VEC;
-    if (row_ok && col < to_len) {
-      Vec<T, VEC> o;
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(x[it][j] * coef);
-      store_vec<T, VEC>(srow + col, o);
+        for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(x[r][it][j] * coef);
+        store_vec<T, VEC>(srow + col, o);
+      }
     }
   }
 }
@@ -282,9 +305,19 @@ __global__ __launch_bounds__(kBlock) void softmax_block(T* __restrict__ score, c
 template <typename T, int VEC, int G, int ITERS>
 static int launch_softmax_rows(T* score, const float* mask, int64_t rows, int heads, int from_len, int to_len,
                                int mask_is_2d, float scale, hipStream_t s) {
-  constexpr int ROWS = kBlock / G;
-  hipLaunchKernelGGL((softmax_rows<T, VEC, G, ITERS>), dim3((unsigned)ceil_div(rows, ROWS)), dim3(kBlock), 0,
-                     s, score, mask, rows, heads, from_len, to_len, mask_is_2d, scale);
+  constexpr int R = ITERS == 1 ? 4 : (ITERS == 2 ? 2 : 1);
+  constexpr int GROUPS = kBlock / G;
+  const dim3 grid((unsigned)ceil_div(rows, (int64_t)GROUPS * R));
+  // vector loads of the fp32 mask need every mask row to start 4*VEC-byte aligned
+  const bool mask_vec = mask != nullptr && (to_len % VEC == 0) &&
+                        (reinterpret_cast<uintptr_t>(mask) % (sizeof(float) * VEC) == 0);
+  if (mask_vec) {
+    hipLaunchKernelGGL((softmax_rows<T, VEC, G, ITERS, R, true>), grid, dim3(kBlock), 0, s, score, mask, rows, heads,
+                       from_len, to_len, mask_is_2d, scale);
+  } else {
+    hipLaunchKernelGGL((softmax_rows<T, VEC, G, ITERS, R, false>), grid, dim3(kBlock), 0, s, score, mask, rows, heads,
+                       from_len, to_len, mask_is_2d, scale);
+  }
   return launch_status("softmax_rows");
 }
 

@@ -281,6 +281,10 @@ TTMI_API int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, i
  *   `scale_dev` is a DEVICE float[2]: [0] receives the scale, [1] is scratch for the max.
  * ttmi_gemm_i8: C_i32[M,N] = A_i8[M,K] * B_i8[N,K]^T.
  * ttmi_dequant_bias: out[m,n] = acc[m,n] * (*act_scale) * w_scale[n] + bias[n] (fp32 out; bias may be NULL). */
+/* ttmi_quantize_weight_rows_i8: per-output-channel symmetric scales for a weight w[N,K] (fp32):
+ *   scales[n] = max_k |w[n,k]| / 127 (1 if the row is zero), q[n,k] = clamp(rint(w[n,k]/scales[n]), -127, 127). */
+TTMI_API int ttmi_quantize_weight_rows_i8(const float* w, int8_t* q, float* scales, int64_t n, int64_t k,
+                                          void* stream);
 TTMI_API int ttmi_quantize_rows_i8(const float* x, int8_t* q, float* scale_dev, int64_t m, int64_t k,
                                    void* stream);
 TTMI_API int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_t n, int64_t k,

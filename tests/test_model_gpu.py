@@ -348,3 +348,57 @@ def test_caching_allocator_behaviour(tt):
         del big
     finally:
         cxx.set_allocator_device_limit_for_test(0)
+
+
+def _oracle_qlinear(oracle, x, w_in_out):
+    """The int8 Linear scheme stated in oracle.cpp: per-channel int8 weights, per-tensor int8
+    activations, exact int32 accumulation, fp32 dequant (no bias)."""
+    qw, sw = oracle.quantize_weight_i8(np.ascontiguousarray(w_in_out.T))
+    x2 = np.ascontiguousarray(x.reshape(-1, x.shape[-1]))
+    qx, sx = oracle.quantize_tensor_i8(x2)
+    return oracle.dequant_bias(oracle.gemm_i8(qx, qw), sx, sw, None).reshape(x.shape[:-1] + (w_in_out.shape[1], ))
+
+
+def test_quantized_bert_layer_vs_oracle_scheme(tt, oracle):
+    """Quantized BERT-base layer, batch 20 x seq 128 (every Linear int8, softmax / LayerNorm fp32)
+    against the same scheme composed from the oracle's pieces, and against the fp32 layer."""
+    model, cfg = _hf_bert(1, seed=21)
+    layer = model.encoder.layer[0]
+    qlayer = tt.QBertLayer.from_torch(layer)
+    B, S, H, heads = 20, 128, cfg.hidden_size, cfg.num_attention_heads
+    x = torch.randn(B, S, H, generator=torch.Generator().manual_seed(4)).cuda()
+    ext = torch.zeros(B, 1, 1, S)
+    ext[3, ..., 100:] = -10000.0
+    ext = ext.cuda()
+    got = host(qlayer(x, ext)[0])
+
+    w = oracle_layer_weights({k: v.detach().cpu().numpy() for k, v in layer.named_parameters()})
+    xn, d = host(x), H // heads
+    qkv = _oracle_qlinear(oracle, xn, w["qkv_w"])
+    q, k, v = oracle.split_add_bias_transpose(qkv, w["qkv_b"], B, S, heads, d)
+    prob = oracle.apply_mask_and_softmax(oracle.batch_matmul(q, k, True, 1.0 / np.sqrt(d)), host(ext), 1.0, True)
+    merged = oracle.transpose_for_score(oracle.batch_matmul(prob, v, False)).reshape(B, S, H)
+    a = oracle.add_bias_layer_norm(_oracle_qlinear(oracle, merged, w["attn_out_w"]), xn, w["attn_out_b"], w["attn_ln_g"],
+                                   w["attn_ln_b"])
+    inter = oracle.add_bias_act(_oracle_qlinear(oracle, a, w["inter_w"]), w["inter_b"], 0)
+    want = oracle.add_bias_layer_norm(_oracle_qlinear(oracle, inter, w["out_w"]), a, w["out_b"], w["out_ln_g"], w["out_ln_b"])
+    # identical integer arithmetic; fp32 differences upstream (1e-7) can move an activation across a
+    # rounding boundary, i.e. one int8 step in one element, hence not bit-exact end to end: almost
+    # all elements agree to fp32 accuracy and the rare flipped step stays small
+    diff = np.abs(got - want)
+    assert float(diff.mean()) < 2e-5 and float((diff > 1e-4).mean()) < 0.02 and diff.max() < 5e-2
+    with torch.no_grad():
+        fp32 = layer(x, attention_mask=ext)
+    fp32 = host(fp32[0] if isinstance(fp32, tuple) else fp32)
+    assert max_abs(got, fp32) < 0.15 and float(np.abs(got - fp32).mean()) < 0.01
+
+
+def test_quantized_bert_model_runs_and_tracks_fp32(tt):
+    model, cfg = _hf_bert(12, seed=22)
+    qmodel = tt.QBertModel.from_torch(model, backend="turbo")
+    ids = torch.randint(0, cfg.vocab_size, (20, 128), generator=torch.Generator().manual_seed(5)).cuda()
+    with torch.no_grad():
+        want = model(input_ids=ids).last_hidden_state
+    seq, pooled = qmodel(ids)[:2]
+    assert seq.shape == (20, 128, cfg.hidden_size) and pooled.shape == (20, cfg.hidden_size)
+    assert float((seq - want).abs().mean()) < 0.03  # int8 noise through 12 layers, not a parity bound

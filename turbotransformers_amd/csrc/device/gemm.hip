@@ -353,7 +353,10 @@ __device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], 
   }
 }
 
-template <typename T, int BM, int BN, int WM, int WN, bool B_KN, bool ALIGNED, typename Epi>
+// DEPTH = number of K steps prefetched into registers ahead of the one being computed (1 or 2).
+// Small tiles are latency-bound (one step of MFMA work is shorter than a global load), so the
+// 64x64 configuration keeps two steps in flight.
+template <typename T, int BM, int BN, int WM, int WN, bool B_KN, bool ALIGNED, int DEPTH, typename Epi>
 __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g, const Epi epi) {
   constexpr int NT = WM * WN * kWave;
   constexpr int KPC = 16 / sizeof(T);          // elements per chunk
@@ -393,7 +396,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  Chunk ra[A_ITERS], rb[B_ITERS];
+  Chunk ra[DEPTH][A_ITERS], rb[DEPTH][B_ITERS];
 
   auto load_chunk = [&](const T* base, int64_t ld, int row, int row_limit, int kcol, int k_limit) -> Chunk {
     // 16 bytes of row `row`, elements kcol..kcol+KPC-1; zero outside [0,row_limit) x [0,k_limit)
@@ -412,7 +415,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
     return c;
   };
 
-  auto load_global = [&](int kt) {
+  auto load_global = [&](int kt, Chunk (&ra)[A_ITERS], Chunk (&rb)[B_ITERS]) {
     const int k0 = kt * BK;
 #pragma unroll
     for (int i = 0; i < A_ITERS; ++i) {
@@ -431,7 +434,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
     }
   };
 
-  auto store_lds = [&](int stage) {
+  auto store_lds = [&](int stage, const Chunk (&ra)[A_ITERS], const Chunk (&rb)[B_ITERS]) {
     char* as = smem + stage * STAGE;
     char* bs = as + A_BYTES;
 #pragma unroll
@@ -485,15 +488,33 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
   };
 
   const int ksteps = (g.k + BK - 1) / BK;
-  load_global(0);
-  store_lds(0);
+  load_global(0, ra[0], rb[0]);
+  store_lds(0, ra[0], rb[0]);
   __syncthreads();
-  for (int kt = 0; kt < ksteps; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < ksteps) load_global(kt + 1);
-    compute(cur);
-    if (kt + 1 < ksteps) store_lds(cur ^ 1);
-    __syncthreads();
+  if (DEPTH == 1) {
+    for (int kt = 0; kt < ksteps; ++kt) {
+      const int cur = kt & 1;
+      if (kt + 1 < ksteps) load_global(kt + 1, ra[0], rb[0]);
+      compute(cur);
+      if (kt + 1 < ksteps) store_lds(cur ^ 1, ra[0], rb[0]);
+      __syncthreads();
+    }
+  } else {
+    // register slot s%2 holds K step s+1; loads past the last step return zero chunks without
+    // touching memory.  Unrolled by two so that the slot index is a compile-time constant.
+    load_global(1, ra[0], rb[0]);
+    load_global(2, ra[DEPTH - 1], rb[DEPTH - 1]);
+    auto step = [&](int kt, Chunk (&sa)[A_ITERS], Chunk (&sb)[B_ITERS]) {
+      const int cur = kt & 1;
+      compute(cur);
+      store_lds(cur ^ 1, sa, sb);      // step kt+1
+      __syncthreads();
+      load_global(kt + 3, sa, sb);     // refill the slot just drained
+    };
+    for (int kt = 0; kt < ksteps; kt += 2) {
+      step(kt, ra[0], rb[0]);
+      if (kt + 1 < ksteps) step(kt + 1, ra[DEPTH - 1], rb[DEPTH - 1]);
+    }
   }
 
   store_tile<T, TM, TN, NT, 2 * STAGE>(acc, smem, epi, g, z, m0 + wm0, n0 + wn0, lane, wave);
@@ -667,7 +688,8 @@ static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
   TTMI_REQUIRE(tiles < (1ll << 30) && batch < 65536, "GEMM grid too large");
   const unsigned grid_x = (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd);
-  auto kern = gemm_kernel<T, BM, BN, WM, WN, B_KN, ALIGNED, Epi>;
+  constexpr int DEPTH = (BM * BN <= 64 * 64 && ALIGNED) ? 2 : 1;
+  auto kern = gemm_kernel<T, BM, BN, WM, WN, B_KN, ALIGNED, DEPTH, Epi>;
   if (LDS > 64 * 1024) {
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {

@@ -52,6 +52,25 @@ __global__ __launch_bounds__(256) void dequant_bias_kernel(const int32_t* __rest
   }
 }
 
+// Per-output-channel symmetric weight quantisation: one wavefront per row of w[N,K].
+__global__ __launch_bounds__(256) void quantize_weight_rows_kernel(const float* __restrict__ w, int8_t* __restrict__ q,
+                                                                   float* __restrict__ scales, int64_t n, int64_t k) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / kWave;
+  if (row >= n) return;
+  const int lane = threadIdx.x % kWave;
+  const float* wr = w + row * k;
+  float mx = 0.f;
+  for (int64_t c = lane; c < k; c += kWave) mx = fmaxf(mx, fabsf(wr[c]));
+  mx = group_max<kWave>(mx);
+  const float scale = mx > 0.f ? mx / 127.0f : 1.0f;
+  if (lane == 0) scales[row] = scale;
+  for (int64_t c = lane; c < k; c += kWave) {
+    float r = rintf(wr[c] / scale);
+    r = fminf(fmaxf(r, -127.f), 127.f);
+    q[row * k + c] = (int8_t)r;
+  }
+}
+
 __global__ void token_rows_kernel(const int32_t* __restrict__ cu, int batch, int max_seq, int total,
                                   int32_t* __restrict__ rows) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
@@ -82,6 +101,14 @@ int ttmi_quantize_rows_i8(const float* x, int8_t* q, float* scale_dev, int64_t m
   hipLaunchKernelGGL(absmax_kernel, dim3(flat_grid(n)), dim3(256), 0, s, x, n, reinterpret_cast<uint32_t*>(scale_dev + 1));
   hipLaunchKernelGGL(quantize_kernel, dim3(flat_grid(n)), dim3(256), 0, s, x, q, scale_dev, n);
   return launch_status("quantize_rows_i8");
+}
+
+int ttmi_quantize_weight_rows_i8(const float* w, int8_t* q, float* scales, int64_t n, int64_t k, void* stream) {
+  TTMI_REQUIRE(w && q && scales, "null tensor");
+  if (n * k <= 0) return 0;
+  hipLaunchKernelGGL(quantize_weight_rows_kernel, dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, (hipStream_t)stream, w, q,
+                     scales, n, k);
+  return launch_status("quantize_weight_rows_i8");
 }
 
 int ttmi_dequant_bias(const int32_t* acc, const float* act_scale_dev, const float* w_scale, const float* bias,

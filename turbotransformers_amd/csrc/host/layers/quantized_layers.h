@@ -1,0 +1,56 @@
+// int8 Linear layers for the quantized BERT configuration: int8 weights with symmetric
+// per-output-channel scales, int8 activations with one dynamic scale per call (max|x| over the
+// whole [tokens, in] activation), int32 accumulation on v_mfma_i32_32x32x32_i8, fp32 dequant.
+// Softmax and LayerNorm stay fp32.
+//
+// In the reference the int8 GEMM is not C++ at all: QBertIntermediate / QBertOutput wrap
+// torch.quantization.quantize_dynamic modules (python/turbo_transformers/layers/qmodeling_bert.py:17,35)
+// and only the fused fp32 epilogues are turbo kernels.  The classes here keep that split
+// (QuantizedLinear has no bias; FusedAddBiasGELU / FusedAddBiasLayerNorm follow it) and add
+// QuantizedBertAttention so that every Linear of the layer is int8.
+#pragma once
+
+#include <mutex>
+
+#include "core/tensor.h"
+
+namespace turbo_transformers {
+namespace layers {
+
+class QuantizedLinear {
+ public:
+  // weight: fp32 [in, out] (the layout every other layer takes); quantized on first use.
+  explicit QuantizedLinear(core::Tensor weight) : weight_(std::move(weight)) {}
+  // output[tokens, out] (fp32) = dequant(q(input) * q(weight)^T); no bias.
+  void operator()(const core::Tensor& input_tensor, core::Tensor* output_tensor) const;
+  int64_t in_features() const { return weight_.shape(0); }
+  int64_t out_features() const { return weight_.shape(1); }
+
+ private:
+  void Prepare() const;
+  core::Tensor weight_;
+  mutable core::Tensor q_weight_, w_scales_, q_input_, acc_, act_scale_;
+  mutable bool prepared_ = false;
+};
+
+class QuantizedBertAttention {
+ public:
+  QuantizedBertAttention(core::Tensor qkv_weight, core::Tensor qkv_bias, core::Tensor dense_weight, core::Tensor dense_bias,
+                         core::Tensor layer_norm_weight, core::Tensor layer_norm_bias, int64_t num_attention_heads)
+      : qkv_(std::move(qkv_weight)), dense_(std::move(dense_weight)), qkv_bias_(std::move(qkv_bias)),
+        dense_bias_(std::move(dense_bias)), ln_weight_(std::move(layer_norm_weight)), ln_bias_(std::move(layer_norm_bias)),
+        heads_(num_attention_heads) {}
+  // Same contract as BertAttention::operator() for fp32 tensors.
+  void operator()(const core::Tensor& input_tensor, const core::Tensor& attention_mask, core::Tensor* output,
+                  core::Tensor* attn = nullptr) const;
+
+ private:
+  QuantizedLinear qkv_, dense_;
+  core::Tensor qkv_bias_, dense_bias_, ln_weight_, ln_bias_;
+  int64_t heads_;
+  mutable core::Tensor qkv_out_, q_, k_, v_, ctx_, merged_, score_scratch_;
+  mutable std::mutex mutex_;
+};
+
+}  // namespace layers
+}  // namespace turbo_transformers

@@ -16,6 +16,7 @@
 #include "core/tensor.h"
 #include "layers/bert_layers.h"
 #include "layers/multi_headed_attention.h"
+#include "layers/quantized_layers.h"
 #include "loaders/npz_load.h"
 #include "ttmi.h"
 
@@ -195,6 +196,18 @@ PYBIND11_MODULE(turbo_transformers_cxx, m) {
   py::class_<layers::LinearBias>(m, "LinearBias")
       .def(py::init([](Tensor& w, Tensor& b) { return new layers::LinearBias(std::move(w), std::move(b)); }))
       .def("__call__", &layers::LinearBias::operator());
+
+  py::class_<layers::QuantizedLinear>(m, "QuantizedLinear")
+      .def(py::init([](Tensor& w) { return new layers::QuantizedLinear(std::move(w)); }))
+      .def("__call__", &layers::QuantizedLinear::operator());
+
+  py::class_<layers::QuantizedBertAttention>(m, "QuantizedBertAttention")
+      .def(py::init([](Tensor& qkv_w, Tensor& qkv_b, Tensor& dense_w, Tensor& dense_b, Tensor& ln_w, Tensor& ln_b, int heads) {
+        return new layers::QuantizedBertAttention(std::move(qkv_w), std::move(qkv_b), std::move(dense_w), std::move(dense_b),
+                                                  std::move(ln_w), std::move(ln_b), heads);
+      }))
+      .def("__call__", &layers::QuantizedBertAttention::operator(), py::arg("input_tensor"), py::arg("attention_mask"),
+           py::arg("output"), py::arg("attn") = nullptr);
 
   m.def("build_smart_pad_mask",
         [](const std::vector<int64_t>& lens, Tensor* out) {

@@ -4,11 +4,13 @@ from .modeling_smart_pad import (MultiHeadedAttentionSmartBatch, BertLayerSmartB
                                  BertModelNoPoolerSmartBatch, BertModelSmartBatch)
 from .modeling_albert import (AlbertEmbeddings, AlbertAttention, AlbertLayer, AlbertLayerGroup, AlbertTransformer,
                               AlbertModel)
+from .qmodeling_bert import QBertIntermediate, QBertOutput, QBertAttention, QBertLayer, QBertEncoder, QBertModel
 from .return_type import ReturnType
 
 __all__ = [
     'BertEmbeddings', 'BertIntermediate', 'BertOutput', 'BertAttention', 'BertLayer', 'BertEncoder', 'BertModel',
     'BertModelNoPooler', 'ReturnType', 'BertPooler', 'SequencePool', 'PoolingType', 'MultiHeadedAttentionSmartBatch',
     'BertLayerSmartBatch', 'BertEncoderSmartBatch', 'BertModelNoPoolerSmartBatch', 'BertModelSmartBatch',
+    'QBertIntermediate', 'QBertOutput', 'QBertAttention', 'QBertLayer', 'QBertEncoder', 'QBertModel',
     'AlbertEmbeddings', 'AlbertAttention', 'AlbertLayer', 'AlbertLayerGroup', 'AlbertTransformer', 'AlbertModel',
 ]

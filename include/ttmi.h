@@ -244,11 +244,14 @@ TTMI_API int ttmi_gemm_batched_heads(const void* a, const void* b, void* c, int6
  * It replaces BatchMatMul + ApplyMaskAndSoftmax + BatchMatMul + TransposeForScore
  * (layers/multi_headed_attention.cpp:323-354) when the [B,h,S,S] probabilities are not an
  * output: the score tensor never reaches HBM.  With `cu_seqlens` (device int32 [B+1]) q,k,v are
- * the zero-padded tensors of a packed batch (S = max length): keys and queries >= len[b] are
- * skipped and `out` is packed [sum(len), h*64] (…smart_batch.cpp:368-392). */
+ * the padded tensors of a packed batch (S = max length): keys and queries >= len[b] are never
+ * read (pad rows need not be zero) and `out` is packed [sum(len), h*64]
+ * (…smart_batch.cpp:368-392).  `v_seq_pitch` = 0: v is [B,h,S,64]; > 0: v is stored transposed,
+ * [B,h,64,v_seq_pitch] with v_seq_pitch a multiple of 8 and >= S, the layout the QKV_SPLIT
+ * epilogues write when asked to (the faster path: tiles of V^T are copied, not scattered). */
 TTMI_API int ttmi_fused_attention(const void* q, const void* k, const void* v, const float* mask, void* out,
                                   const int32_t* cu_seqlens, int64_t batch, int64_t heads, int64_t seq,
-                                  int64_t head_dim, float scale, int dtype, void* stream);
+                                  int64_t head_dim, int64_t v_seq_pitch, float scale, int dtype, void* stream);
 
 /* Arguments of the fused epilogues; unused members are NULL / 0. */
 typedef struct ttmi_epilogue_args {
@@ -261,6 +264,8 @@ typedef struct ttmi_epilogue_args {
   int64_t head_dim;          /* d; N must equal 3*h*d                                       */
   const int32_t* token_rows; /* device [M]: packed token -> b*max_seq+s (QKV_SPLIT_PAD)      */
   int64_t batch;             /* B                                   (QKV_SPLIT_PAD)          */
+  int64_t v_seq_pitch;       /* 0: v is [B,h,S,d]; > 0: v is written transposed as
+                                [B,h,d,v_seq_pitch] (multiple of 8, >= seq)  (QKV_SPLIT*)    */
 } ttmi_epilogue_args;
 
 /* MatMul with the following memory-bound op folded into the store of the accumulators:

@@ -151,8 +151,11 @@ def test_fused_bias_and_bias_residual(ttmi, oracle, dt):
 
 
 @pytest.mark.parametrize("dt", ALL_DTYPES)
-@pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 7, 2, 32)])
-def test_fused_qkv_split(ttmi, oracle, dt, B, S, h, d):
+@pytest.mark.parametrize("v_transposed", [False, True])
+@pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 7, 2, 32), (2, 300, 16, 64), (5, 13, 3, 64)])
+def test_fused_qkv_split(ttmi, oracle, dt, B, S, h, d, v_transposed):
+    """QKV GEMM + SplitAddBiasTransposeForScore; with v_seq_pitch the V third lands transposed,
+    [B,h,d,pitch] (pad columns untouched), everything else as before."""
     import ctypes
     rng = np.random.default_rng(S)
     H = h * d
@@ -160,20 +163,29 @@ def test_fused_qkv_split(ttmi, oracle, dt, B, S, h, d):
     bias = rng.standard_normal(3 * H).astype(np.float32)
     dA, dW, db = dev(A, dt), dev(W, dt), dev(bias, dt)
     q, k, v = (torch.empty((B, h, S, d), dtype=dA.dtype, device="cuda") for _ in range(3))
-    args = _epi(bias=db, q=q, k=k, v=v, seq=S, heads=h, head_dim=d)
+    pitch = (S + 7) // 8 * 8 + 8 if v_transposed else 0
+    if v_transposed:
+        v = torch.full((B, h, d, pitch), 7.0, dtype=dA.dtype, device="cuda")
+    args = _epi(bias=db, q=q, k=k, v=v, seq=S, heads=h, head_dim=d, v_seq_pitch=pitch)
     ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), None, B * S, 3 * H, H, H, H, 3 * H, capi.EPI_QKV_SPLIT,
                             ctypes.byref(args), TTMI_DTYPES[dt], stream()))
     qkv = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
     want = oracle.split_add_bias_transpose(qkv, rounded(bias, dt), B, S, h, d)
-    for got, w in zip((q, k, v), want):
-        assert max_abs(host(got), w) <= GEMM_TOL[dt] * 2
+    got_v = host(v)
+    if v_transposed:
+        assert np.all(got_v[..., S:] == 7.0)
+        got_v = got_v[..., :S].transpose(0, 1, 3, 2)
+    for got, w in zip((host(q), host(k), got_v), want):
+        assert max_abs(got, w) <= GEMM_TOL[dt] * 2
 
 
 @pytest.mark.parametrize("dt", ALL_DTYPES)
-def test_fused_qkv_split_pad(ttmi, oracle, dt):
+@pytest.mark.parametrize("v_transposed", [False, True])
+@pytest.mark.parametrize("lens", [[9, 30, 1, 17], [64, 8, 200, 16, 33]])
+def test_fused_qkv_split_pad(ttmi, oracle, dt, lens, v_transposed):
     import ctypes
     rng = np.random.default_rng(21)
-    lens = np.array([9, 30, 1, 17], np.int64)
+    lens = np.array(lens, np.int64)
     h, d = 4, 64
     H, B, maxS, total = h * d, len(lens), int(lens.max()), int(lens.sum())
     A, W = _ab(rng, total, 3 * H, H, 1)
@@ -184,13 +196,19 @@ def test_fused_qkv_split_pad(ttmi, oracle, dt):
     rows = torch.empty(total, dtype=torch.int32, device="cuda")
     ok(ttmi.ttmi_build_token_rows(ptr(dev(cu)), B, maxS, total, ptr(rows), stream()))
     q, k, v = (torch.zeros((B, h, maxS, d), dtype=dA.dtype, device="cuda") for _ in range(3))
-    args = _epi(bias=db, q=q, k=k, v=v, seq=maxS, heads=h, head_dim=d, token_rows=rows, batch=B)
+    pitch = (maxS + 7) // 8 * 8 if v_transposed else 0
+    if v_transposed:
+        v = torch.zeros((B, h, d, pitch), dtype=dA.dtype, device="cuda")
+    args = _epi(bias=db, q=q, k=k, v=v, seq=maxS, heads=h, head_dim=d, token_rows=rows, batch=B, v_seq_pitch=pitch)
     ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), None, total, 3 * H, H, H, H, 3 * H, capi.EPI_QKV_SPLIT_PAD,
                             ctypes.byref(args), TTMI_DTYPES[dt], stream()))
     qkv = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
     want = oracle.split_add_bias_transpose_pad(qkv, rounded(bias, dt), lens, h, d)
-    for got, w in zip((q, k, v), want):
-        assert max_abs(host(got), w) <= GEMM_TOL[dt] * 2
+    got_v = host(v)
+    if v_transposed:
+        got_v = got_v[..., :maxS].transpose(0, 1, 3, 2)
+    for got, w in zip((host(q), host(k), got_v), want):
+        assert max_abs(got, w) <= GEMM_TOL[dt] * 2
 
 
 @pytest.mark.parametrize("M,N,K", [(20, 768, 768), (2560, 3072, 768), (2560, 768, 3072), (33, 48, 80), (300, 1000, 130)])
@@ -231,10 +249,23 @@ def test_int8_linear_pipeline(ttmi, oracle):
     assert max_abs(want, x @ w.T + bias) < 0.05  # and the scheme itself approximates the fp32 Linear
 
 
+def _v_operand(V, dt, v_transposed, poison=True):
+    """-> (device tensor, v_seq_pitch).  The transposed form is [B,h,d,pitch]; its pad columns hold
+    NaN so that a kernel that lets them reach the output fails the comparison."""
+    if not v_transposed:
+        return dev(V, dt), 0
+    B, h, S, d = V.shape
+    pitch = (S + 7) // 8 * 8
+    vt = np.full((B, h, d, pitch), np.nan if poison else 0.0, np.float32)
+    vt[..., :S] = V.transpose(0, 1, 3, 2)
+    return dev(vt, dt), pitch
+
+
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("v_transposed", [False, True])
 @pytest.mark.parametrize("B,h,S,masked", [(2, 3, 128, True), (1, 2, 512, False), (3, 2, 100, True), (2, 1, 37, True),
                                          (1, 1, 500, True), (2, 12, 64, False), (1, 2, 1, False), (1, 1, 700, True)])
-def test_fused_attention_vs_unfused_oracle(ttmi, oracle, dt, B, h, S, masked):
+def test_fused_attention_vs_unfused_oracle(ttmi, oracle, dt, B, h, S, masked, v_transposed):
     """One-kernel softmax(scale QK^T + mask) V against the oracle's four-step chain
     (BatchMatMul, ApplyMaskAndSoftmax, BatchMatMul, TransposeForScore)."""
     rng = np.random.default_rng(S + B)
@@ -245,10 +276,11 @@ def test_fused_attention_vs_unfused_oracle(ttmi, oracle, dt, B, h, S, masked):
         mask = np.zeros((B, 1, 1, S), np.float32)
         mask[0, ..., S // 2 + 1:] = -10000.0
         mask[-1, ..., :S // 3] = -10000.0
-    dQ, dK, dV = dev(Q, dt), dev(K, dt), dev(V, dt)
+    dQ, dK = dev(Q, dt), dev(K, dt)
+    dV, pitch = _v_operand(V, dt, v_transposed)
     out = torch.full((B, S, h * d), 9.0, dtype=dQ.dtype, device="cuda")
     ok(ttmi.ttmi_fused_attention(ptr(dQ), ptr(dK), ptr(dV), ptr(dev(mask)) if masked else None, ptr(out), None, B, h, S, d,
-                                 0.125, TTMI_DTYPES[dt], stream()))
+                                 pitch, 0.125, TTMI_DTYPES[dt], stream()))
     score = oracle.batch_matmul(rounded(Q, dt), rounded(K, dt), True, 0.125)
     prob = oracle.apply_mask_and_softmax(score, mask, 1.0, True)
     want = oracle.transpose_for_score(oracle.batch_matmul(prob, rounded(V, dt), False)).reshape(B, S, h * d)
@@ -257,19 +289,25 @@ def test_fused_attention_vs_unfused_oracle(ttmi, oracle, dt, B, h, S, masked):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
-def test_fused_attention_packed_batch(ttmi, oracle, dt):
+@pytest.mark.parametrize("v_transposed", [False, True])
+def test_fused_attention_packed_batch(ttmi, oracle, dt, v_transposed):
+    """Packed batch: pad rows of q,k,v hold NaN on the device -- the kernel must never let a row
+    past a sequence's length reach the output -- and zeros in the oracle's padded chain."""
     rng = np.random.default_rng(17)
     lens, h, d = [70, 5, 129, 33], 2, 64
     B, maxS, total = len(lens), max(lens), sum(lens)
     Q, K, V = (rng.standard_normal((B, h, maxS, d), np.float32) for _ in range(3))
-    for b, L in enumerate(lens):  # pad rows are zero in the real pipeline
+    Qp, Kp, Vp = Q.copy(), K.copy(), V.copy()
+    for b, L in enumerate(lens):
         Q[b, :, L:], K[b, :, L:], V[b, :, L:] = 0, 0, 0
+        Qp[b, :, L:], Kp[b, :, L:], Vp[b, :, L:] = np.nan, np.nan, np.nan
     cu = np.zeros(B + 1, np.int32)
     cu[1:] = np.cumsum(lens)
     mask = np.where(np.arange(maxS)[None, :] < np.array(lens)[:, None], 0.0, -1e9).astype(np.float32)
     out = torch.full((total, h * d), 9.0, dtype=dev(Q, dt).dtype, device="cuda")
-    ok(ttmi.ttmi_fused_attention(ptr(dev(Q, dt)), ptr(dev(K, dt)), ptr(dev(V, dt)), ptr(dev(mask)), ptr(out), ptr(dev(cu)), B, h,
-                                 maxS, d, 0.125, TTMI_DTYPES[dt], stream()))
+    dV, pitch = _v_operand(Vp, dt, v_transposed)
+    ok(ttmi.ttmi_fused_attention(ptr(dev(Qp, dt)), ptr(dev(Kp, dt)), ptr(dV), ptr(dev(mask)), ptr(out), ptr(dev(cu)), B, h,
+                                 maxS, d, pitch, 0.125, TTMI_DTYPES[dt], stream()))
     score = oracle.batch_matmul(rounded(Q, dt), rounded(K, dt), True, 0.125)
     prob = oracle.apply_mask_and_softmax(score, mask.reshape(B, 1, 1, maxS), 1.0, True)
     ctx = oracle.batch_matmul(prob, rounded(V, dt), False)

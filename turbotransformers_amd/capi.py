@@ -28,7 +28,7 @@ class EpilogueArgs(ctypes.Structure):
         ("bias", ctypes.c_void_p), ("residual", ctypes.c_void_p), ("act", ctypes.c_int),
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
         ("seq", ctypes.c_int64), ("heads", ctypes.c_int64), ("head_dim", ctypes.c_int64),
-        ("token_rows", ctypes.c_void_p), ("batch", ctypes.c_int64),
+        ("token_rows", ctypes.c_void_p), ("batch", ctypes.c_int64), ("v_seq_pitch", ctypes.c_int64),
     ]
 
 

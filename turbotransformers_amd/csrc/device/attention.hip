@@ -6,8 +6,10 @@
 // 4*T*H elements instead of ~2*B*h*S^2).
 //
 // Work split: one workgroup = 4 wavefronts = 128 query rows of one (batch, head); a wavefront
-// owns 32 queries.  K/V advance in tiles of 64 keys staged in LDS (K row-major and
-// XOR-swizzled like the GEMM operands, V transposed to [d][key]).
+// owns 32 queries.  K/V advance in tiles of 64 keys staged in LDS: K row-major [key][d], V
+// transposed [d][key], both in 128-byte rows XOR-swizzled like the GEMM operands.  V may be
+// given already transposed ([B,h,d,pitch], written that way by the QKV GEMM epilogue); then a
+// V tile is copied in 8-byte pieces, otherwise it is scattered element by element.
 //
 // MFMA formulation (v_mfma_f32_32x32x16): scores are computed TRANSPOSED,
 //     St[key, query] = K_tile[key, :] . Q[query, :]      (A = K from LDS, B = Q from registers)
@@ -17,7 +19,8 @@
 //     Ot[d, query] += Vt[d, keys] . Pt[keys, query]      (A = V^T from LDS, B = P from registers)
 // because accumulator registers 8kk..8kk+7 of a lane are exactly the 8 keys that half-wave
 // feeds to MFMA kk.  No cross-lane shuffles of P, no LDS round trip for P.
-// exp() is evaluated as exp2 with log2(e) folded into the scale and the mask.
+// exp() is evaluated as exp2; the mask (divided by the scale) seeds the score accumulators and
+// scale*log2(e) is applied inside the exp2 argument, so no separate scale/mask pass exists.
 #include "common.h"
 
 namespace ttmi {
@@ -25,6 +28,9 @@ namespace ttmi {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4), may_alias));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2), may_alias));
 
 struct __attribute__((may_alias)) alignas(16) Chunk16 {
   uint32_t w[4];
@@ -44,32 +50,60 @@ __device__ __forceinline__ floatx16 mma16<bf16>(const Chunk16& a, const Chunk16&
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// Two floats -> one packed register (round to nearest even): v_cvt_pk_{f16,bf16}_f32.
 template <typename T>
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  const T a = from_float<T>(lo), b = from_float<T>(hi);
-  uint16_t ua, ub;
-  __builtin_memcpy(&ua, &a, 2);
-  __builtin_memcpy(&ub, &b, 2);
-  return (uint32_t)ua | ((uint32_t)ub << 16);
+__device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t pack2<f16>(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{lo, hi}, halfx2));
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<bf16>(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{lo, hi}, bf16x2));
+}
+
+// acc + lo + hi of a packed pair (v_dot2c_f32_*): the softmax denominator is summed from the
+// ROUNDED probabilities, the same values the P.V MFMA consumes.
+template <typename T>
+__device__ __forceinline__ float add_pair(uint32_t p, float acc);
+template <>
+__device__ __forceinline__ float add_pair<f16>(uint32_t p, float acc) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2, p), halfx2{(_Float16)1.0f, (_Float16)1.0f}, acc, false);
+}
+template <>
+__device__ __forceinline__ float add_pair<bf16>(uint32_t p, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, p), bf16x2{(__bf16)1.0f, (__bf16)1.0f}, acc, false);
 }
 
 constexpr int kD = 64;          // head dim
 constexpr int kBQ = 128;        // queries per workgroup
 constexpr int kBKV = 64;        // keys per LDS tile
-constexpr int kVtPitch = kBKV + 4;  // halfs per V^T row (8-byte aligned rows, spreads banks)
 constexpr float kNegBig = -1.0e30f;
 
-template <typename T, bool PACKED>
-__global__ __launch_bounds__(256) void fused_attention_kernel(const T* __restrict__ q, const T* __restrict__ k,
-                                                              const T* __restrict__ v, const float* __restrict__ mask,
-                                                              T* __restrict__ out, const int32_t* __restrict__ cu,
-                                                              int heads, int seq, float scale_log2e) {
+// Position of a key inside its group of 16 in an LDS V^T row.  A lane of the P.V MFMA holds the
+// probabilities of keys {4h..4h+3, 8+4h..8+4h+3} (h = lane/32) of the group; storing the group as
+// [0-3, 8-11, 4-7, 12-15] makes those 8 keys one 16-byte read.
+__device__ __forceinline__ int vt_pos(int within16) {
+  return (within16 & 3) | ((within16 & 4) << 1) | ((within16 & 8) >> 1);
+}
+
+template <typename T, bool PACKED, bool VT>
+__global__ __launch_bounds__(256, 2) void fused_attention_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                                 const T* __restrict__ v, const float* __restrict__ mask,
+                                                                 T* __restrict__ out, const int32_t* __restrict__ cu,
+                                                                 int heads, int seq, int v_pitch, float scale_log2e,
+                                                                 float inv_scale) {
   // one LDS block: [2 x K tile | 2 x V^T tile | 2 x mask]; the front is reused for the output tile
-  constexpr int kKBytes = kBKV * 128, kVtBytes = kD * kVtPitch * (int)sizeof(T);
+  constexpr int kKBytes = kBKV * 128, kVtBytes = kD * 128;
   __shared__ __align__(16) char smem[2 * kKBytes + 2 * kVtBytes + 2 * kBKV * 4];
   static_assert(4 * 32 * (kD + 8) * sizeof(T) <= 2 * kKBytes + 2 * kVtBytes, "output staging must fit in the tile buffers");
   auto k_lds = [&](int stage) { return smem + stage * kKBytes; };
-  auto vt_lds = [&](int stage) { return reinterpret_cast<T*>(smem + 2 * kKBytes + stage * kVtBytes); };
+  auto vt_lds = [&](int stage) { return smem + 2 * kKBytes + stage * kVtBytes; };
+  // additive mask per key, already divided by the score scale: it seeds the score accumulators
   auto mask_lds = [&](int stage) { return reinterpret_cast<float*>(smem + 2 * kKBytes + 2 * kVtBytes) + stage * kBKV; };
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -87,7 +121,7 @@ __global__ __launch_bounds__(256) void fused_attention_kernel(const T* __restric
 
   const T* qb = q + (int64_t)bh * seq * kD;
   const T* kb = k + (int64_t)bh * seq * kD;
-  const T* vb = v + (int64_t)bh * seq * kD;
+  const T* vb = v + (int64_t)bh * kD * (VT ? v_pitch : seq);
 
   // Q fragments: B operand, lane = (query lrow, k-chunk by lhalf); 4 MFMA k-steps cover d = 64.
   Chunk16 qf[4];
@@ -107,99 +141,154 @@ __global__ __launch_bounds__(256) void fused_attention_kernel(const T* __restric
     for (int e = 0; e < 16; ++e) ot[t][e] = 0.f;
   float m_run = kNegBig, l_run = 0.f;
 
-  auto load_tile = [&](int tile, int stage) {
+  // K/V tiles are register-staged: the global loads of tile t+1 are issued before the MFMAs of
+  // tile t and written to the other LDS stage afterwards, so their latency hides behind compute.
+  // Loads past the last key are clamped to valid memory: such keys carry a -1e30 mask, so a
+  // duplicated K row is harmless; V^T columns past the last key may be uninitialised memory and
+  // are zeroed on the way to LDS (0 * NaN would poison the output).
+  // (Named vector registers, not arrays: an array captured by the two lambdas ends up in scratch.)
+  u32x4 kreg0, kreg1, vreg0, vreg1;
+  float mreg = 0.f;
+  auto load_regs = [&](int tile) {
     const int key0 = tile * kBKV;
-    // K: 64 keys x 8 chunks; thread c -> (key c>>3, chunk c&7): 128-byte rows, coalesced
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int c = tid + i * 256;
-      const int key = c >> 3, ch = c & 7;
-      Chunk16 x{{0u, 0u, 0u, 0u}};
-      if (key0 + key < kv_len) x = *reinterpret_cast<const Chunk16*>(kb + (int64_t)(key0 + key) * kD + ch * 8);
-      *reinterpret_cast<Chunk16*>(k_lds(stage) + key * 128 + ((ch ^ ((key >> 1) & 7)) << 4)) = x;
+    const int ch = tid & 7, r0 = tid >> 3;  // chunk and row of this lane's first 16-byte piece; second: row + 32
+    {
+      const T* p0 = kb + (int64_t)min(key0 + r0, kv_len - 1) * kD + ch * 8;  // 128-byte K rows, coalesced
+      const T* p1 = kb + (int64_t)min(key0 + r0 + 32, kv_len - 1) * kD + ch * 8;
+      kreg0 = *reinterpret_cast<const u32x4*>(p0);
+      kreg1 = *reinterpret_cast<const u32x4*>(p1);
     }
-    // V: thread -> (key tid&63, d-chunk (tid>>6) + 4i); scattered into V^T[d][key] so that lanes
-    // write consecutive halfs of one row (no bank conflicts)
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int key = tid & 63, dch = (tid >> 6) + 4 * i;
-      Vec<T, 8> x;
-      if (key0 + key < kv_len) {
-        x = load_vec<T, 8>(vb + (int64_t)(key0 + key) * kD + dch * 8);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x.v[j] = from_float<T>(0.f);
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) vt_lds(stage)[(dch * 8 + j) * kVtPitch + key] = x.v[j];
+    if (VT) {
+      const int ks = min(key0 + ch * 8, v_pitch - 8);
+      vreg0 = *reinterpret_cast<const u32x4*>(vb + (int64_t)r0 * v_pitch + ks);
+      vreg1 = *reinterpret_cast<const u32x4*>(vb + (int64_t)(r0 + 32) * v_pitch + ks);
+    } else {
+      const int key = min(key0 + (tid & 63), kv_len - 1), dch = tid >> 6;
+      vreg0 = *reinterpret_cast<const u32x4*>(vb + (int64_t)key * kD + dch * 8);
+      vreg1 = *reinterpret_cast<const u32x4*>(vb + (int64_t)key * kD + (dch + 4) * 8);
     }
     if (tid < kBKV) {
       const int key = key0 + tid;
-      float mv = kNegBig;
-      if (key < kv_len) mv = mask ? mask[(int64_t)b * seq + key] * 1.4426950408889634f : 0.f;
-      mask_lds(stage)[tid] = mv;
+      const float mv = mask ? mask[(int64_t)b * seq + min(key, kv_len - 1)] * inv_scale : 0.f;
+      mreg = key < kv_len ? mv : kNegBig;
+    }
+  };
+  auto put_vt = [&](u32x4 x, int tile, int stage, int drow, int ch) {
+    if (tile * kBKV + kBKV > kv_len) {  // only the last tile: zero the keys past the end
+      const int nv = kv_len - (tile * kBKV + ch * 8);  // valid keys in this chunk
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        if (2 * w >= nv) x[w] = 0u;
+        else if (2 * w + 1 >= nv) x[w] &= 0xffffu;
+      }
+    }
+    // keys 8ch..8ch+3 and 8ch+4..8ch+7 go to the two 16-byte slots of their 16-key group
+    char* row = vt_lds(stage) + drow * 128 + (ch & 1) * 8;
+    const int slot = (ch >> 1) * 2, sw = (drow >> 1) & 7;
+    *reinterpret_cast<u32x2*>(row + ((slot ^ sw) << 4)) = u32x2{x[0], x[1]};
+    *reinterpret_cast<u32x2*>(row + (((slot + 1) ^ sw) << 4)) = u32x2{x[2], x[3]};
+  };
+  auto scatter_v = [&](u32x4 x, int stage, int dch) {
+    const int key = tid & 63;
+    const int pos = vt_pos(key & 15), slot = (key >> 4) * 2 + (pos >> 3);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int drow = dch * 8 + j;
+      const uint32_t word = x[j >> 1];
+      *reinterpret_cast<uint16_t*>(vt_lds(stage) + drow * 128 + ((slot ^ ((drow >> 1) & 7)) << 4) + (pos & 7) * 2) =
+          (uint16_t)((j & 1) ? (word >> 16) : (word & 0xffffu));
+    }
+  };
+  auto store_tile_lds = [&](int tile, int stage) {
+    const int ch = tid & 7, r0 = tid >> 3;
+    *reinterpret_cast<u32x4*>(k_lds(stage) + r0 * 128 + ((ch ^ ((r0 >> 1) & 7)) << 4)) = kreg0;
+    *reinterpret_cast<u32x4*>(k_lds(stage) + (r0 + 32) * 128 + ((ch ^ ((r0 >> 1) & 7)) << 4)) = kreg1;  // +32 keeps the swizzle
+    if (VT) {
+      put_vt(vreg0, tile, stage, r0, ch);
+      put_vt(vreg1, tile, stage, r0 + 32, ch);
+    } else {
+      scatter_v(vreg0, stage, tid >> 6);
+      scatter_v(vreg1, stage, (tid >> 6) + 4);
+    }
+    if (tid < kBKV) mask_lds(stage)[tid] = mreg;
+  };
+
+  // One 64-key tile from LDS stage STAGE (a compile-time constant so every LDS address is a
+  // per-lane base plus an immediate).  m_run is kept in raw score units; the softmax scale and
+  // log2(e) are applied inside the exp2 argument: p = exp2(s*c - m*c), c = scale*log2(e).
+  const int k_lane = lrow * 128, k_sw = (lrow >> 1) & 7;
+  int k_off[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) k_off[kk] = k_lane + (((2 * kk + lhalf) ^ k_sw) << 4);  // rows +32 keep the swizzle
+  auto compute_tile = [&](auto stage_c) {
+    constexpr int STAGE = decltype(stage_c)::value;
+    const char* kt = smem + STAGE * kKBytes;
+    const char* vt = smem + 2 * kKBytes + STAGE * kVtBytes;
+    const float* mk = reinterpret_cast<const float*>(smem + 2 * kKBytes + 2 * kVtBytes) + STAGE * kBKV;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {  // two 32-key sub-tiles
+      const int sk = sub * 32;
+      // st[e] = score of (key sk + 8*(e/4) + 4*lhalf + e%4, query lrow), seeded with mask/scale
+      floatx16 st;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float4 mv = *reinterpret_cast<const float4*>(mk + sk + 8 * g + 4 * lhalf);
+        st[4 * g] = mv.x, st[4 * g + 1] = mv.y, st[4 * g + 2] = mv.z, st[4 * g + 3] = mv.w;
+      }
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const Chunk16 kf = *reinterpret_cast<const Chunk16*>(kt + sk * 128 + k_off[kk]);
+        st = mma16<T>(kf, qf[kk], st);
+      }
+      float mx = st[0];
+#pragma unroll
+      for (int e = 1; e < 16; ++e) mx = fmaxf(mx, st[e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+      const float neg_m = -m_new * scale_log2e;
+      m_run = m_new;
+      Chunk16 pf[2];
+      float psum = 0.f;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[2 * w], scale_log2e, neg_m));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[2 * w + 1], scale_log2e, neg_m));
+        const uint32_t pk = pack2<T>(p0, p1);
+        pf[w >> 2].w[w & 3] = pk;
+        psum = add_pair<T>(pk, psum);
+      }
+      l_run = l_run * alpha + psum;
+      if (__any(alpha != 1.0f)) {  // the running maximum rarely moves after the first tiles
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) ot[t][e] *= alpha;
+      }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const Chunk16 vf = *reinterpret_cast<const Chunk16*>(vt + t * 32 * 128 + k_off[2 * sub + kk]);
+          ot[t] = mma16<T>(vf, pf[kk], ot[t]);
+        }
     }
   };
 
   const int tiles = (kv_len + kBKV - 1) / kBKV;
   const bool wave_active = q0 < q_len;
-  load_tile(0, 0);
+  load_regs(0);
+  store_tile_lds(0, 0);
   __syncthreads();
-  for (int tile = 0; tile < tiles; ++tile) {
-    const int stage = tile & 1;
-    if (tile + 1 < tiles) load_tile(tile + 1, stage ^ 1);
-    if (wave_active) {
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {  // two 32-key sub-tiles
-        const int sk = sub * 32;
-        floatx16 st;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) st[e] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          const int key = sk + lrow;
-          const Chunk16 kf = *reinterpret_cast<const Chunk16*>(k_lds(stage) + key * 128 + (((2 * kk + lhalf) ^ ((key >> 1) & 7)) << 4));
-          st = mma16<T>(kf, qf[kk], st);
-        }
-        // st[e] = score of (key sk + 8*(e/4) + 4*lhalf + e%4, query lrow)
-        float mx = kNegBig;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int key = sk + 8 * (e / 4) + 4 * lhalf + (e % 4);
-          st[e] = st[e] * scale_log2e + mask_lds(stage)[key];
-          mx = fmaxf(mx, st[e]);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          st[e] = __builtin_amdgcn_exp2f(st[e] - m_new);
-          psum += st[e];
-        }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) ot[t][e] *= alpha;
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          Chunk16 pf;
-#pragma unroll
-          for (int w = 0; w < 4; ++w) pf.w[w] = pack2<T>(st[8 * kk + 2 * w], st[8 * kk + 2 * w + 1]);
-#pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            const T* row = vt_lds(stage) + (t * 32 + lrow) * kVtPitch + sk + 16 * kk + 4 * lhalf;
-            const Chunk8 lo = *reinterpret_cast<const Chunk8*>(row);
-            const Chunk8 hi = *reinterpret_cast<const Chunk8*>(row + 8);
-            const Chunk16 vf{{lo.w[0], lo.w[1], hi.w[0], hi.w[1]}};
-            ot[t] = mma16<T>(vf, pf, ot[t]);
-          }
-        }
-      }
-    }
+  for (int tile = 0; tile < tiles; tile += 2) {
+    if (tile + 1 < tiles) load_regs(tile + 1);
+    if (wave_active) compute_tile(std::integral_constant<int, 0>{});
+    if (tile + 1 < tiles) store_tile_lds(tile + 1, 1);
+    __syncthreads();
+    if (tile + 1 >= tiles) break;
+    if (tile + 2 < tiles) load_regs(tile + 2);
+    if (wave_active) compute_tile(std::integral_constant<int, 1>{});
+    if (tile + 2 < tiles) store_tile_lds(tile + 2, 0);
     __syncthreads();
   }
 
@@ -237,25 +326,34 @@ extern "C" {
 
 int ttmi_fused_attention(const void* q, const void* k, const void* v, const float* mask, void* out,
                          const int32_t* cu_seqlens, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
-                         float scale, int dtype, void* stream) {
+                         int64_t v_seq_pitch, float scale, int dtype, void* stream) {
   TTMI_REQUIRE(q && k && v && out, "null tensor");
   TTMI_REQUIRE(head_dim == kD, "fused attention is built for head_dim 64");
   TTMI_REQUIRE(dtype == TTMI_F16 || dtype == TTMI_BF16, "fused attention is built for fp16 / bf16");
   TTMI_REQUIRE(batch > 0 && heads > 0 && seq > 0 && batch * heads < 65536 && seq < (1 << 24), "bad shape");
+  TTMI_REQUIRE(v_seq_pitch == 0 || (v_seq_pitch >= seq && v_seq_pitch % 8 == 0 && v_seq_pitch < (1 << 24)),
+               "v_seq_pitch must be 0 or a multiple of 8 that is >= seq");
+  TTMI_REQUIRE(scale > 0.f, "scale must be positive");
   uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                    reinterpret_cast<uintptr_t>(out);
   TTMI_REQUIRE((bits & 15) == 0, "tensors must be 16-byte aligned");
   const dim3 grid((unsigned)ceil_div(seq, kBQ), (unsigned)(batch * heads));
-  const float sl2 = scale * 1.4426950408889634f;
+  const float sl2 = scale * 1.4426950408889634f, inv_scale = 1.0f / scale;
   hipStream_t s = (hipStream_t)stream;
-#define TTMI_FA_LAUNCH(T, PACKED)                                                                              \
-  hipLaunchKernelGGL((fused_attention_kernel<T, PACKED>), grid, dim3(256), 0, s, (const T*)q, (const T*)k,     \
-                     (const T*)v, mask, (T*)out, cu_seqlens, (int)heads, (int)seq, sl2)
+#define TTMI_FA_LAUNCH(T, PACKED, VT)                                                                            \
+  hipLaunchKernelGGL((fused_attention_kernel<T, PACKED, VT>), grid, dim3(256), 0, s, (const T*)q, (const T*)k,   \
+                     (const T*)v, mask, (T*)out, cu_seqlens, (int)heads, (int)seq, (int)v_seq_pitch, sl2, inv_scale)
+#define TTMI_FA_LAYOUT(T, PACKED)                                          \
+  do {                                                                     \
+    if (v_seq_pitch) TTMI_FA_LAUNCH(T, PACKED, true);                      \
+    else TTMI_FA_LAUNCH(T, PACKED, false);                                 \
+  } while (0)
   if (dtype == TTMI_F16) {
-    if (cu_seqlens) TTMI_FA_LAUNCH(f16, true); else TTMI_FA_LAUNCH(f16, false);
+    if (cu_seqlens) TTMI_FA_LAYOUT(f16, true); else TTMI_FA_LAYOUT(f16, false);
   } else {
-    if (cu_seqlens) TTMI_FA_LAUNCH(bf16, true); else TTMI_FA_LAUNCH(bf16, false);
+    if (cu_seqlens) TTMI_FA_LAYOUT(bf16, true); else TTMI_FA_LAYOUT(bf16, false);
   }
+#undef TTMI_FA_LAYOUT
 #undef TTMI_FA_LAUNCH
   return launch_status("fused_attention");
 }

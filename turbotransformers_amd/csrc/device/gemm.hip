@@ -254,7 +254,35 @@ struct EpiQkvSplit {
   int seq, heads, dim, hidden;
   FastDiv div_seq, div_hidden, div_dim;
   bool vec;
+  int v_pitch;  // 0: v is [B,h,S,d]; > 0: v is written transposed, [B,h,d,v_pitch]
   __device__ __forceinline__ Bias8 prepare(int n, int n_limit) const { return load_bias8<T>(bias, n, n_limit, vec); }
+  // Columns of the V third are stored by the column pass when V is kept transposed.
+  __device__ __forceinline__ bool column_pass() const { return v_pitch > 0; }
+  __device__ __forceinline__ int first_column_of_pass() const { return 2 * hidden; }
+  // Rows m..m+7 of output column n (n in the V third): eight consecutive sequence positions of
+  // one V^T row when they belong to one sequence, one 16-byte store.
+  __device__ __forceinline__ void store_col8(int m, int m_limit, int n, float (&val)[8]) const {
+    const uint32_t rem = (uint32_t)(n - 2 * hidden);
+    const uint32_t head = div_dim.div(rem);
+    const uint32_t i = rem - head * dim;
+    const float bv = to_float(bias[n]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) val[j] += bv;
+    const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;  // b*seq + s
+    const uint32_t b = div_seq.div(prow);
+    const uint32_t s = prow - b * seq;
+    bool fast = m + 8 <= m_limit && (s & 7u) == 0 && s + 8 <= (uint32_t)seq;
+    if (PAD && fast) fast = (uint32_t)token_rows[m + 7] == prow + 7;
+    if (fast) {
+      store_row8<T>(v + (((int64_t)b * heads + head) * dim + i) * v_pitch + s, val);
+      return;
+    }
+    for (int j = 0; j < 8 && m + j < m_limit; ++j) {
+      const uint32_t pr = PAD ? (uint32_t)token_rows[m + j] : (uint32_t)(m + j);
+      const uint32_t bj = div_seq.div(pr);
+      v[(((int64_t)bj * heads + head) * dim + i) * v_pitch + (pr - bj * seq)] = from_float<T>(val[j]);
+    }
+  }
   __device__ __forceinline__ T* dest(uint32_t b, uint32_t s, uint32_t n) const {
     const uint32_t w = div_hidden.div(n);
     const uint32_t rem = n - w * hidden;
@@ -264,6 +292,7 @@ struct EpiQkvSplit {
     return base + (((int64_t)b * heads + head) * seq + s) * dim + i;
   }
   __device__ __forceinline__ void store8(int, int m, int n, float (&val)[8], int valid, const Bias8& bs) const {
+    if (v_pitch > 0 && n >= 2 * hidden) return;  // left to the column pass (groups of 8 never straddle 2*hidden)
     const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;  // b*seq + s
     const uint32_t b = div_seq.div(prow);
     const uint32_t s = prow - b * seq;
@@ -307,11 +336,18 @@ struct EpiInt32 {
 // 256-byte bank period: slot = (r&1)*8 + physical chunk, with physical chunk = chunk ^ ((r>>1)&7).
 __device__ __forceinline__ int swizzle(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
 
+template <typename Epi>
+struct HasColumnPass : std::false_type {};
+template <typename T, bool PAD>
+struct HasColumnPass<EpiQkvSplit<T, PAD>> : std::true_type {};
+
 // Epilogue shared by the kernels.  acc[i][j][e] is C[row 8*(e/4) + 4*lhalf + e%4][col lrow] of its
 // 32x32 block.  Each wavefront stages one 32-row strip of its sub-tile at a time in its own
 // slice of LDS (the K-loop buffers are free after the last barrier), then reads it back
 // row-major, 8 columns per lane, so that global stores are full 16-byte vectors in 128-byte
-// row segments.
+// row segments.  An epilogue with a column pass (transposed V of the QKV split) gets the
+// columns from first_column_of_pass() on read back column-major instead: 8 rows of one column
+// per lane, four adjacent lanes covering 32 consecutive rows = 64 contiguous output bytes.
 template <typename T, int TM, int TN, int NT, int LDS_BYTES, typename Epi>
 __device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], char* smem, const Epi& epi,
                                            const GemmArgs& g, int z, int wave_m0, int wave_n0, int lane, int wave) {
@@ -329,8 +365,31 @@ __device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], 
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = acc[i][j][e];
+    bool row_pass = true;
+    if constexpr (HasColumnPass<Epi>::value) {
+      if (epi.column_pass()) {
+        const int first = epi.first_column_of_pass();
+        row_pass = wave_n0 < first;  // wave-uniform
+        if (wave_n0 + W > first) {
+          constexpr int CPASSES = 4 * W / kWave;
+#pragma unroll
+          for (int p = 0; p < CPASSES; ++p) {
+            const int idx = p * kWave + lane;
+            const int rg = idx & 3, c = idx >> 2;
+            const int m = wave_m0 + i * 32 + rg * 8, ncol = wave_n0 + c;
+            if (m < g.m && ncol < g.n && ncol >= first) {
+              AccScalar v[8];
+#pragma unroll
+              for (int t = 0; t < 8; ++t) v[t] = stage[(rg * 8 + t) * LDW + c];
+              epi.store_col8(m, g.m, ncol, v);
+            }
+          }
+        }
+      }
+    }
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
+      if (!row_pass) break;
       const int idx = p * kWave + lane;          // (row, column group) handled by this lane
       const int r = idx / LANES_PER_ROW, cg = idx % LANES_PER_ROW;
       if (r >= 32) continue;
@@ -909,15 +968,18 @@ int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n,
         if (pad) TTMI_REQUIRE(args->token_rows != nullptr && args->batch > 0, "padded QKV epilogue needs token_rows and batch");
         else TTMI_REQUIRE(m % args->seq == 0, "M must be a multiple of seq");
         const int hidden = (int)(args->heads * args->head_dim);
+        const int64_t vp = args->v_seq_pitch;
+        TTMI_REQUIRE(vp == 0 || (vp >= args->seq && vp % 8 == 0 && vp < (1ll << 31) && hidden % 8 == 0),
+                     "v_seq_pitch must be 0 or a multiple of 8 that is >= seq (hidden a multiple of 8)");
         if (pad) {
           EpiQkvSplit<T, true> epi{(T*)args->q, (T*)args->k, (T*)args->v, (const T*)args->bias, args->token_rows,
                                    (int)args->seq, (int)args->heads, (int)args->head_dim, hidden,
-                                   FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim), qkv_vec};
+                                   FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim), qkv_vec, (int)vp};
           return (launch_gemm<T, false>(g, epi, 1, aligned, s));
         }
         EpiQkvSplit<T, false> epi{(T*)args->q, (T*)args->k, (T*)args->v, (const T*)args->bias, nullptr,
                                   (int)args->seq, (int)args->heads, (int)args->head_dim, hidden,
-                                  FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim), qkv_vec};
+                                  FastDiv((uint32_t)args->seq), FastDiv((uint32_t)hidden), FastDiv((uint32_t)args->head_dim), qkv_vec, (int)vp};
         return (launch_gemm<T, false>(g, epi, 1, aligned, s));
       }
       default:

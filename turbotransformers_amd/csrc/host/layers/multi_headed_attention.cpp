@@ -34,10 +34,21 @@ void BertAttention::EnforceShapeAndType() const {
   TT_ENFORCE_EQ(layernorm_beta_.numel(), dense_weight_.shape(0), "LayerNorm bias size mismatch");
 }
 
+bool MultiHeadedAttention::UseFusedCore(const Tensor& attention_mask, const Tensor* att_score, int64_t head_dim, int dtype) {
+  bool mask_is_key_mask = true;
+  if (!attention_mask.is_null()) {
+    mask_is_key_mask = attention_mask.n_dim() == 2 || (attention_mask.n_dim() == 3 && attention_mask.shape(1) == 1) ||
+                       (attention_mask.n_dim() == 4 && attention_mask.shape(2) == 1);
+  }
+  return att_score == nullptr && head_dim == 64 && (dtype == TTMI_F16 || dtype == TTMI_BF16) && mask_is_key_mask;
+}
+
+static int64_t RoundUp8(int64_t n) { return (n + 7) / 8 * 8; }
+
 // score -> softmax -> P V -> merge heads -> output projection -> bias (+input) (+LayerNorm)
 void MultiHeadedAttention::SelfAttentionTail(const Tensor& query_tensor, const Tensor& attention_mask, Tensor* output,
                                              Tensor* att_score, int64_t batch, int64_t seq,
-                                             const std::vector<int64_t>* seq_list, bool post_layernorm,
+                                             const std::vector<int64_t>* seq_list, int64_t v_pitch, bool post_layernorm,
                                              bool post_add_input, bool is_trans_weight) const {
   const int dt = kernels::DeviceDType(query_tensor);
   const DLDeviceType dev = query_tensor.device_type();
@@ -49,14 +60,8 @@ void MultiHeadedAttention::SelfAttentionTail(const Tensor& query_tensor, const T
   const float scaler = 1.0f / std::sqrt(static_cast<float>(d));
 
   // Nobody asked for the probabilities: run the whole core as one kernel; the [B,h,S,S] scores
-  // never reach HBM.  (fp16/bf16, head size 64, key mask broadcast over query rows.)
-  bool mask_is_key_mask = true;
-  if (!attention_mask.is_null()) {
-    mask_is_key_mask = attention_mask.n_dim() == 2 || (attention_mask.n_dim() == 3 && attention_mask.shape(1) == 1) ||
-                       (attention_mask.n_dim() == 4 && attention_mask.shape(2) == 1);
-  }
-  const bool fused_core = att_score == nullptr && d == 64 && (dt == TTMI_F16 || dt == TTMI_BF16) && mask_is_key_mask;
-  if (fused_core) {
+  // never reach HBM.
+  if (v_pitch > 0) {
     const float* mask = nullptr;
     if (!attention_mask.is_null()) {
       TT_ENFORCE_EQ(attention_mask.numel(), batch * seq, "attention mask has the wrong size");
@@ -65,7 +70,7 @@ void MultiHeadedAttention::SelfAttentionTail(const Tensor& query_tensor, const T
     const int32_t* cu = nullptr;
     if (seq_list != nullptr) cu = DeviceContext::GetInstance().GetSeqPlan(*seq_list).cu_seqlens;
     TT_DEVICE_CALL(ttmi_fused_attention(q_.raw(), k_.raw(), v_.raw(), mask, ctx_.mutable_raw(), cu, batch, heads, seq, d,
-                                        scaler, dt, Stream()));
+                                        v_pitch, scaler, dt, Stream()));
   } else {
   Tensor* score = att_score != nullptr ? att_score : &score_scratch_;
   score->ReshapeAs(query_tensor.dtype(), {batch, heads, seq, seq}, dev, dev_id, "batch_gemm3/Reshape");
@@ -137,9 +142,12 @@ void MultiHeadedAttention::operator()(const Tensor& key_tensor, const Tensor& va
     qkv_in = &ln_query_;
   }
 
+  // with the fused core V is kept transposed, [B,h,d,pitch]: its tiles are then plain copies
+  const int64_t v_pitch = UseFusedCore(attention_mask, att_score, d, dt) ? RoundUp8(seq) : 0;
   q_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/q/Reshape");
   k_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/k/Reshape");
-  v_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/v/Reshape");
+  if (v_pitch > 0) v_.ReshapeAs(query_tensor.dtype(), {batch, heads, d, v_pitch}, dev, dev_id, "self/v/Reshape");
+  else v_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/v/Reshape");
   // gemm012_fused + SplitAddBiasTransposeForScore in one launch (:199-203)
   ttmi_epilogue_args args{};
   args.bias = qkv_bias_.raw();
@@ -149,11 +157,12 @@ void MultiHeadedAttention::operator()(const Tensor& key_tensor, const Tensor& va
   args.seq = seq;
   args.heads = heads;
   args.head_dim = d;
+  args.v_seq_pitch = v_pitch;
   TT_DEVICE_CALL(ttmi_gemm_fused(qkv_in->raw(), qkv_packed_.Get(qkv_weight_, is_trans_weight), nullptr, batch * seq, 3 * hidden,
                                  hidden, hidden, hidden, 3 * hidden, TTMI_EPI_QKV_SPLIT, &args, dt, Stream()));
 
-  SelfAttentionTail(query_tensor, attention_mask, output, att_score, batch, seq, nullptr, post_layernorm, post_add_input,
-                    is_trans_weight);
+  SelfAttentionTail(query_tensor, attention_mask, output, att_score, batch, seq, nullptr, v_pitch, post_layernorm,
+                    post_add_input, is_trans_weight);
 }
 
 void BertAttention::operator()(const Tensor& input_tensor, const Tensor& attention_mask, Tensor* output, Tensor* attn,
@@ -195,12 +204,16 @@ void MultiHeadedAttentionSmartBatch::operator()(const Tensor& key_tensor, const 
   const int dev_id = query_tensor.device_id();
   const int64_t batch = plan.batch, max_seq = plan.max_seq;
 
-  // Zero-padded q,k,v: pad rows stay exactly 0 (transpose.cpp:504-522), then the QKV GEMM
-  // scatters bias-added rows of the packed input into them.
+  // Padded q,k,v; the QKV GEMM scatters bias-added rows of the packed input into them.  The
+  // unfused core multiplies whole padded tensors, so pad rows must be exactly 0 there
+  // (transpose.cpp:504-522); the fused kernel never reads a pad row, so nothing is cleared.
+  const int64_t v_pitch = UseFusedCore(attention_mask, att_score, d, dt) ? RoundUp8(max_seq) : 0;
   Tensor* qkv[3] = {&q_, &k_, &v_};
   const char* names[3] = {"self/q/Reshape", "self/k/Reshape", "self/v/Reshape"};
   for (int i = 0; i < 3; ++i) {
-    qkv[i]->ReshapeAs(query_tensor.dtype(), {batch, heads, max_seq, d}, dev, dev_id, names[i]);
+    if (i == 2 && v_pitch > 0) qkv[i]->ReshapeAs(query_tensor.dtype(), {batch, heads, d, v_pitch}, dev, dev_id, names[i]);
+    else qkv[i]->ReshapeAs(query_tensor.dtype(), {batch, heads, max_seq, d}, dev, dev_id, names[i]);
+    if (v_pitch > 0) continue;
     const size_t bytes = (size_t)qkv[i]->numel() * qkv[i]->element_size();
     TT_DEVICE_CALL(ttmi_memset_zero(qkv[i]->mutable_raw(), (bytes + 3) / 4 * 4  /* capacity is rounded to 512 B */, Stream()));
   }
@@ -214,11 +227,12 @@ void MultiHeadedAttentionSmartBatch::operator()(const Tensor& key_tensor, const 
   args.head_dim = d;
   args.token_rows = plan.token_rows;
   args.batch = batch;
+  args.v_seq_pitch = v_pitch;
   TT_DEVICE_CALL(ttmi_gemm_fused(query_tensor.raw(), qkv_packed_.Get(qkv_weight_, is_trans_weight), nullptr, plan.total,
                                  3 * hidden, hidden, hidden, hidden, 3 * hidden, TTMI_EPI_QKV_SPLIT_PAD, &args, dt, Stream()));
 
-  SelfAttentionTail(query_tensor, attention_mask, output, att_score, batch, max_seq, &query_seq_len_list, post_layernorm,
-                    post_add_input, is_trans_weight);
+  SelfAttentionTail(query_tensor, attention_mask, output, att_score, batch, max_seq, &query_seq_len_list, v_pitch,
+                    post_layernorm, post_add_input, is_trans_weight);
 }
 
 }  // namespace layers

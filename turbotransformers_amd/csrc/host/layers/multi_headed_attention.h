@@ -60,9 +60,13 @@ class MultiHeadedAttention {
 
  protected:
   // Everything after q/k/v exist, shared by the dense and the smart-batch layers.
+  // `v_pitch` > 0: v_ holds V transposed, [B,h,d,v_pitch], and the fused attention kernel runs.
   void SelfAttentionTail(const core::Tensor& query_tensor, const core::Tensor& attention_mask, core::Tensor* output,
                          core::Tensor* att_score, int64_t batch, int64_t seq, const std::vector<int64_t>* seq_list,
-                         bool post_layernorm, bool post_add_input, bool is_trans_weight) const;
+                         int64_t v_pitch, bool post_layernorm, bool post_add_input, bool is_trans_weight) const;
+  // The whole attention core runs as one kernel when nobody asks for the probabilities
+  // (fp16/bf16, head size 64, additive key mask broadcast over the query rows).
+  static bool UseFusedCore(const core::Tensor& attention_mask, const core::Tensor* att_score, int64_t head_dim, int dtype);
 
   core::Tensor k_weight_, k_bias_, v_weight_, v_bias_, q_weight_, q_bias_;
   core::Tensor dense_weight_, dense_bias_, qkv_weight_, qkv_bias_;

@@ -73,14 +73,19 @@ __device__ __forceinline__ float group_max(float v) {
 }
 
 // tanh-form GELU exactly as the reference states it, written through the logistic identity
-// 0.5*(1+tanh(u)) == 1/(1+exp(-2u)) so it costs one v_exp_f32 and one v_rcp_f32.
+// 0.5*(1+tanh(u)) == 1/(1+exp(-2u)), u = sqrt(2/pi)*(x + 0.044715 x^3).  With the constants folded
+// into one polynomial in x it is 5 VALU operations plus one v_exp_f32 and one v_rcp_f32 (both
+// accurate to 1 ulp; a correctly rounded division would cost ten more instructions).
 __device__ __forceinline__ float gelu_tanh(float x) {
-  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  return x * __frcp_rn(1.0f + __expf(-2.0f * u));
+  constexpr float c1 = -2.0f * 1.4426950408889634f * 0.7978845608028654f;  // exp(-2u) = exp2(x*(c1 + c3 x^2))
+  constexpr float c3 = c1 * 0.044715f;
+  const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(x * x, c3, c1));
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 __device__ __forceinline__ float fast_tanh(float x) {
   // tanh(x) = 1 - 2/(exp(2x)+1); saturates cleanly at +-1 when exp overflows/underflows
-  return 1.0f - 2.0f * __frcp_rn(__expf(2.0f * x) + 1.0f);
+  const float e = __builtin_amdgcn_exp2f(x * (2.0f * 1.4426950408889634f));
+  return __builtin_fmaf(-2.0f, __builtin_amdgcn_rcpf(e + 1.0f), 1.0f);
 }
 
 template <int ACT>

@@ -48,6 +48,7 @@ __device__ __forceinline__ Chunk pack_chunk(const T (&tmp)[N]) {
 constexpr int kRowBytes = 128;   // bytes of K per LDS row and per K step
 constexpr int kChunks = 8;       // 16-byte chunks per LDS row
 constexpr int kNumXcd = 8;
+constexpr int kLdsPerCu = 160 * 1024;
 
 template <typename T>
 struct Mma;
@@ -155,24 +156,17 @@ __device__ __forceinline__ void load_row8(const T* p, float (&v)[8]) {
   }
 }
 
-// Per-lane column state of an epilogue: the 8 bias values of the lane's columns.
-struct Bias8 {
-  float b[8];
-};
-
-template <typename T>
-__device__ __forceinline__ Bias8 load_bias8(const T* bias, int n, int n_limit, bool vec) {
-  Bias8 r;
-  if (bias == nullptr) {
+// The bias of an epilogue (bias_ptr(), may be null) is added by store_tile while the values are
+// still in accumulator layout, where a lane owns ONE column per 32x32 block: the kernels fetch
+// those few values at the start of a tile, so their latency never shows.
+template <int TN, typename Epi>
+__device__ __forceinline__ void load_bias_columns(const Epi& epi, int n_first, int n_limit, float (&bj)[TN]) {
+  const auto* bias = epi.bias_ptr();
 #pragma unroll
-    for (int j = 0; j < 8; ++j) r.b[j] = 0.f;
-  } else if (vec && n + 8 <= n_limit) {
-    load_row8<T>(bias + n, r.b);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) r.b[j] = (n + j < n_limit) ? to_float(bias[n + j]) : 0.f;
+  for (int j = 0; j < TN; ++j) {
+    const int n = n_first + j * 32;
+    bj[j] = (bias != nullptr && n < n_limit) ? to_float(bias[n]) : 0.f;
   }
-  return r;
 }
 
 template <typename T>
@@ -183,8 +177,8 @@ struct EpiAlphaBeta {
   int inner;
   float alpha, beta;
   bool vec;
-  __device__ __forceinline__ Bias8 prepare(int, int) const { return Bias8{}; }
-  __device__ __forceinline__ void store8(int z, int m, int n, float (&v)[8], int valid, const Bias8&) const {
+  __device__ __forceinline__ const T* bias_ptr() const { return nullptr; }
+  __device__ __forceinline__ void store8(int z, int m, int n, float (&v)[8], int valid) const {
     T* p = c + (int64_t)(z / inner) * c_outer + (int64_t)(z % inner) * c_inner + (int64_t)m * ldc + n;
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] *= alpha;
@@ -214,13 +208,12 @@ struct EpiBias {
   const T* residual;
   int64_t ldc;
   bool vec;
-  __device__ __forceinline__ Bias8 prepare(int n, int n_limit) const { return load_bias8<T>(bias, n, n_limit, vec); }
-  __device__ __forceinline__ void store8(int, int m, int n, float (&v)[8], int valid, const Bias8& bs) const {
+  __device__ __forceinline__ const T* bias_ptr() const { return bias; }
+  __device__ __forceinline__ void store8(int, int m, int n, float (&v)[8], int valid) const {
     const int64_t off = (int64_t)m * ldc + n;
+    if (HAS_ACT) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      v[j] += bs.b[j];
-      if (HAS_ACT) v[j] = apply_act<ACT>(v[j]);
+      for (int j = 0; j < 8; ++j) v[j] = apply_act<ACT>(v[j]);
     }
     if (vec && valid == 8) {
       if (HAS_RES) {
@@ -255,7 +248,7 @@ struct EpiQkvSplit {
   FastDiv div_seq, div_hidden, div_dim;
   bool vec;
   int v_pitch;  // 0: v is [B,h,S,d]; > 0: v is written transposed, [B,h,d,v_pitch]
-  __device__ __forceinline__ Bias8 prepare(int n, int n_limit) const { return load_bias8<T>(bias, n, n_limit, vec); }
+  __device__ __forceinline__ const T* bias_ptr() const { return bias; }
   // Columns of the V third are stored by the column pass when V is kept transposed.
   __device__ __forceinline__ bool column_pass() const { return v_pitch > 0; }
   __device__ __forceinline__ int first_column_of_pass() const { return 2 * hidden; }
@@ -265,9 +258,6 @@ struct EpiQkvSplit {
     const uint32_t rem = (uint32_t)(n - 2 * hidden);
     const uint32_t head = div_dim.div(rem);
     const uint32_t i = rem - head * dim;
-    const float bv = to_float(bias[n]);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) val[j] += bv;
     const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;  // b*seq + s
     const uint32_t b = div_seq.div(prow);
     const uint32_t s = prow - b * seq;
@@ -291,13 +281,11 @@ struct EpiQkvSplit {
     T* base = (w == 0) ? q : (w == 1 ? k : v);
     return base + (((int64_t)b * heads + head) * seq + s) * dim + i;
   }
-  __device__ __forceinline__ void store8(int, int m, int n, float (&val)[8], int valid, const Bias8& bs) const {
+  __device__ __forceinline__ void store8(int, int m, int n, float (&val)[8], int valid) const {
     if (v_pitch > 0 && n >= 2 * hidden) return;  // left to the column pass (groups of 8 never straddle 2*hidden)
     const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;  // b*seq + s
     const uint32_t b = div_seq.div(prow);
     const uint32_t s = prow - b * seq;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) val[j] += bs.b[j];
     if (vec && valid == 8) {
       store_row8<T>(dest(b, s, (uint32_t)n), val);
     } else {
@@ -311,8 +299,8 @@ struct EpiInt32 {
   int32_t* c;
   int64_t ldc;
   bool vec;
-  __device__ __forceinline__ Bias8 prepare(int, int) const { return Bias8{}; }
-  __device__ __forceinline__ void store8(int, int m, int n, int (&v)[8], int valid, const Bias8&) const {
+  __device__ __forceinline__ const int32_t* bias_ptr() const { return nullptr; }
+  __device__ __forceinline__ void store8(int, int m, int n, int (&v)[8], int valid) const {
     int32_t* p = c + (int64_t)m * ldc + n;
     if (vec && valid == 8) {
       Vec<int32_t, 4> lo, hi;
@@ -349,8 +337,9 @@ struct HasColumnPass<EpiQkvSplit<T, PAD>> : std::true_type {};
 // columns from first_column_of_pass() on read back column-major instead: 8 rows of one column
 // per lane, four adjacent lanes covering 32 consecutive rows = 64 contiguous output bytes.
 template <typename T, int TM, int TN, int NT, int LDS_BYTES, typename Epi>
-__device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], char* smem, const Epi& epi,
-                                           const GemmArgs& g, int z, int wave_m0, int wave_n0, int lane, int wave) {
+__device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], const float (&bj)[TN], char* smem,
+                                           const Epi& epi, const GemmArgs& g, int z, int wave_m0, int wave_n0, int lane,
+                                           int wave) {
   using AccScalar = typename Mma<T>::AccScalar;
   constexpr int W = TN * 32;             // strip width (columns)
   constexpr int LDW = W + 4;             // padded pitch in words: rows stay 16-byte aligned
@@ -364,7 +353,8 @@ __device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], 
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = acc[i][j][e];
+      for (int e = 0; e < 16; ++e)
+        stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = acc[i][j][e] + (AccScalar)bj[j];
     bool row_pass = true;
     if constexpr (HasColumnPass<Epi>::value) {
       if (epi.column_pass()) {
@@ -404,10 +394,7 @@ __device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], 
         v[t] = lo.v[t];
         v[t + 4] = hi.v[t];
       }
-      if (m < g.m && valid > 0) {
-        const Bias8 cstate = epi.prepare(ncol, g.n);
-        epi.store8(z, m, ncol, v, valid, cstate);
-      }
+      if (m < g.m && valid > 0) epi.store8(z, m, ncol, v, valid);
     }
   }
 }
@@ -576,7 +563,9 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
     }
   }
 
-  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, smem, epi, g, z, m0 + wm0, n0 + wn0, lane, wave);
+  float bj[TN];
+  load_bias_columns<TN>(epi, n0 + wn0 + lrow, g.n, bj);
+  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, bj, smem, epi, g, z, m0 + wm0, n0 + wn0, lane, wave);
 }
 
 // ------------------------------------------------------------------ fast-path kernel -----
@@ -590,6 +579,16 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
 //     last valid row (their results are never stored).
 //   * MFMA operand fragments are double-buffered in registers: the LDS reads of k-substep
 //     kk+1 are issued before the MFMAs of kk.
+// LDS bytes of the fast kernel: two K-loop stages, or one stage plus the epilogue staging area
+// (which starts at the second stage and may run past it), whichever is larger.
+template <int BM, int BN, int WM, int WN>
+constexpr int fast_epilogue_bytes() { return WM * WN * 32 * (BN / WN + 4) * 4; }
+template <int BM, int BN, int WM, int WN>
+constexpr int fast_lds_bytes() {
+  constexpr int stage = (BM + BN) * kRowBytes;
+  return stage + (fast_epilogue_bytes<BM, BN, WM, WN>() > stage ? fast_epilogue_bytes<BM, BN, WM, WN>() : stage);
+}
+
 template <typename T, int BM, int BN, int WM, int WN, typename Epi>
 __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmArgs g, const Epi epi) {
   constexpr int NW = WM * WN, NT = NW * kWave;
@@ -604,13 +603,19 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
 
   extern __shared__ __align__(16) char smem[];
 
+  // Persistent workgroups: the grid holds at most as many workgroups as stay resident and each
+  // walks over several tiles.  XCD x owns the contiguous tile range [x*per_xcd, (x+1)*per_xcd);
+  // its workgroups (ids equal to x mod 8) stride through it together.  Between two tiles the
+  // first K step of the next tile is fetched (DMA into stage 0) while the epilogue of the
+  // finished tile runs out of the other half of LDS, and the epilogue's global stores drain
+  // under the next tile's K loop.
   const int tiles = g.tiles_m * g.tiles_n;
   const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
-  const int logical = (int)(blockIdx.x % kNumXcd) * per_xcd + (int)(blockIdx.x / kNumXcd);
-  if (logical >= tiles) return;
-  const int tile_m = logical / g.tiles_n, tile_n = logical % g.tiles_n;
+  const int xcd = (int)(blockIdx.x % kNumXcd), stride = (int)(gridDim.x / kNumXcd);
+  const int xcd_end = min((xcd + 1) * per_xcd, tiles);
+  int logical = xcd * per_xcd + (int)(blockIdx.x / kNumXcd);
+  if (logical >= xcd_end) return;
   const int z = blockIdx.z;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const T* A = reinterpret_cast<const T*>(g.a) + (int64_t)(z / g.inner) * g.a_outer + (int64_t)(z % g.inner) * g.a_inner;
   const T* B = reinterpret_cast<const T*>(g.b) + (int64_t)(z / g.inner) * g.b_outer + (int64_t)(z % g.inner) * g.b_inner;
 
@@ -618,11 +623,17 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   const int lane = tid % kWave, wave = tid / kWave;
   const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
   const int lrow = lane & 31, lhalf = lane >> 5;
+  lds_char* lds0 = reinterpret_cast<lds_char*>(reinterpret_cast<uintptr_t>(smem));
+  // byte offsets of this lane's operand rows inside a stage (swizzle folded in per k-substep)
+  const int a_row0 = (wm0 + lrow) * kRowBytes, b_row0 = A_BYTES + (wn0 + lrow) * kRowBytes;
+  const int swz = ((lrow >> 1) & 7);  // rows wm0 + 32 i + lrow share (row>>1)&7 with lrow
+  const int ksteps = g.k / BK;
 
-  // per-lane source pointers of the DMA loads (advanced by one K step per iteration)
+  // per-lane source pointers of the DMA loads (advanced by one K step per issue)
   const T* pa[A_LOADS];
   const T* pb[B_LOADS];
-  {
+  auto point_at = [&](int tile) {
+    const int m0 = (tile / g.tiles_n) * BM, n0 = (tile % g.tiles_n) * BN;
     const int sub = lane >> 3, p = lane & 7;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
@@ -636,8 +647,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
       const int c = p ^ ((row >> 1) & 7);
       pb[i] = B + (int64_t)min(n0 + row, g.n - 1) * g.ldb + c * KPC;
     }
-  }
-  lds_char* lds0 = reinterpret_cast<lds_char*>(reinterpret_cast<uintptr_t>(smem));
+  };
 
   // The DMA builtin exists only in the device pass; the host pass of this translation unit
   // needs the kernel body just to emit the launch stub.
@@ -660,18 +670,6 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   auto issue = [&](int) { (void)lds0; };
 #endif
 
-  Acc acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-
-  // byte offsets of this lane's operand rows inside a stage (swizzle folded in per k-substep)
-  const int a_row0 = (wm0 + lrow) * kRowBytes, b_row0 = A_BYTES + (wn0 + lrow) * kRowBytes;
-  const int swz = ((lrow >> 1) & 7);  // rows wm0 + 32 i + lrow share (row>>1)&7 with lrow
-
   auto read_frags = [&](const char* st, int kk, Chunk (&fa)[TM], Chunk (&fb)[TN]) {
     const int off = ((2 * kk + lhalf) ^ swz) << 4;
 #pragma unroll
@@ -688,6 +686,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   // so neither the LDS latency nor the barrier leaves the MFMA pipe without queued work.
   // sched_group_barrier pins the interleaving (mask 0x100 = LDS read, 0x008 = MFMA).
   constexpr int READS = TM + TN, MMAS = TM * TN;
+  Acc acc[TM][TN];
   auto mma_step = [&](Chunk (&fa)[TM], Chunk (&fb)[TN]) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -708,33 +707,54 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
     __builtin_amdgcn_sched_group_barrier(0x008, MF - 1 - PER * READS, 0);
   };
 
-  const int ksteps = g.k / BK;
+  point_at(logical);
   issue(0);
-  __syncthreads();
-  if (ksteps > 1) issue(1);
-  Chunk fa[2][TM], fb[2][TN];
-  read_frags(smem, 0, fa[0], fb[0]);
-  for (int kt = 0; kt < ksteps; ++kt) {
-    const int cur = kt & 1;
-    const char* st = smem + cur * STAGE;
-    const char* st_next = smem + (cur ^ 1) * STAGE;
-    read_frags(st, 1, fa[1], fb[1]);
-    mma_step(fa[0], fb[0]);
-    interleave();
-    read_frags(st, 2, fa[0], fb[0]);
-    mma_step(fa[1], fb[1]);
-    interleave();
-    read_frags(st, 3, fa[1], fb[1]);
-    mma_step(fa[0], fb[0]);
-    interleave();
-    __syncthreads();
-    if (kt + 2 < ksteps) issue(cur);
-    read_frags(st_next, 0, fa[0], fb[0]);  // harmless on the last step
-    mma_step(fa[1], fb[1]);
-    interleave();
+  for (;;) {
+    const int m0 = (logical / g.tiles_n) * BM, n0 = (logical % g.tiles_n) * BN;
+    float bj[TN];
+    load_bias_columns<TN>(epi, n0 + wn0 + lrow, g.n, bj);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+    __syncthreads();  // step 0 has landed; the previous tile's staging area has been read out
+    if (ksteps > 1) issue(1);
+    Chunk fa[2][TM], fb[2][TN];
+    read_frags(smem, 0, fa[0], fb[0]);
+    for (int kt = 0; kt < ksteps; ++kt) {
+      const int cur = kt & 1;
+      const char* st = smem + cur * STAGE;
+      const char* st_next = smem + (cur ^ 1) * STAGE;
+      read_frags(st, 1, fa[1], fb[1]);
+      mma_step(fa[0], fb[0]);
+      interleave();
+      read_frags(st, 2, fa[0], fb[0]);
+      mma_step(fa[1], fb[1]);
+      interleave();
+      read_frags(st, 3, fa[1], fb[1]);
+      mma_step(fa[0], fb[0]);
+      interleave();
+      __syncthreads();
+      if (kt + 2 < ksteps) issue(cur);
+      read_frags(st_next, 0, fa[0], fb[0]);  // harmless on the last step
+      mma_step(fa[1], fb[1]);
+      interleave();
+    }
+    __syncthreads();  // all LDS reads of this tile are done
+
+    const int next = logical + stride;
+    if (next < xcd_end) {  // stage 0 is free: fetch the next tile's first K step under the epilogue
+      point_at(next);
+      issue(0);
+    }
+    store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN>() - STAGE>(acc, bj, smem + STAGE, epi, g, z, m0 + wm0, n0 + wn0,
+                                                                         lane, wave);
+    if (next >= xcd_end) break;
+    logical = next;
   }
-  __syncthreads();  // all LDS reads done before the epilogue reuses the buffers
-  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, smem, epi, g, z, m0 + wm0, n0 + wn0, lane, wave);
 }
 
 // ------------------------------------------------------------------------ launching -----
@@ -762,15 +782,28 @@ static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+static int compute_units() {
+  static int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return cus;
+}
+
 template <typename T, int BM, int BN, int WM, int WN, typename Epi>
 static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   constexpr int NT = WM * WN * kWave;
-  constexpr int LDS = 2 * (BM + BN) * kRowBytes;
+  constexpr int LDS = fast_lds_bytes<BM, BN, WM, WN>();
+  static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
   g.tiles_m = (g.m + BM - 1) / BM;
   g.tiles_n = (g.n + BN - 1) / BN;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
   TTMI_REQUIRE(tiles < (1ll << 30) && batch < 65536, "GEMM grid too large");
-  const unsigned grid_x = (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd);
+  // as many workgroups as stay resident (LDS-limited), a multiple of the XCD count
+  const int64_t resident = (int64_t)compute_units() * std::max(1, kLdsPerCu / LDS);
+  const unsigned grid_x = (unsigned)(std::min(ceil_div(tiles, kNumXcd), std::max<int64_t>(1, resident / kNumXcd)) * kNumXcd);
   auto kern = gemm_fast_kernel<T, BM, BN, WM, WN, Epi>;
   if (LDS > 64 * 1024) {
     static bool attr_set = false;  // per instantiation

@@ -119,7 +119,17 @@ def run_smart_batch(steps, warmup):
             "padded": {"ms_per_step": ms_p, "p50_ms": p50_p, "seq_per_s": len(lens) / ms_p * 1e3}}
 
 
-def kernel_rooflines(dtype="f16", batch=64, seq=512, hidden=768, heads=12, ffn=3072, iters=20):
+# HBM-side traffic of one launch in bytes, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
+# `python3 bench.py --pmc-kernel <name>` (counter KiB scaled by what the calibration copy reads: x2.0 for
+# FETCH_SIZE, x1.0 for WRITE_SIZE).  Keyed by (kernel of the roofline pass, dtype, batch, seq).
+MEASURED_TRAFFIC = {
+    ("ffn1_gemm+bias+gelu", "f16", 64, 512): {"fetch_bytes": 141900 * 2.0 * 1024, "write_bytes": 196600 * 1.0 * 1024},
+}
+
+COPY_ELEMS = 64 << 20  # fp32 elements of the calibration copy: reads 256 MiB, writes 256 MiB
+
+
+def kernel_rooflines(dtype="f16", batch=64, seq=512, hidden=768, heads=12, ffn=3072, iters=20, only=None):
     """Each kernel of the layer alone, at its real shape, timed with HIP events on the work stream
     through the C ABI.  GEMMs: algorithmic FLOPs = 2*M*N*K against the MFMA peak; memory-bound
     kernels: algorithmic bytes (each tensor read / written once) against 8 TB/s."""
@@ -146,11 +156,14 @@ def kernel_rooflines(dtype="f16", batch=64, seq=512, hidden=768, heads=12, ffn=3
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / iters * 1e3  # us
 
-    x, w_qkv, w_o, w_1, w_2 = rnd(T, H), rnd(3 * H, H), rnd(H, H), rnd(F, H), rnd(H, F)
+    # operand statistics as in the forward (LayerNorm-scale activations, N(0,0.02) weights): the MFMA
+    # clock under load depends on how many operand bits toggle
+    wgt = lambda *shape: (torch.randn(*shape, device="cuda") * 0.02).to(tdt)
+    x, w_qkv, w_o, w_1, w_2 = rnd(T, H) * 2, wgt(3 * H, H), wgt(H, H), wgt(F, H), wgt(H, F)
     b_qkv, b_h, b_f, gam = rnd(3 * H), rnd(H), rnd(F), rnd(H)
-    q, k, v = (torch.empty(batch, heads, seq, d, device="cuda", dtype=tdt) for _ in range(3))
+    q, k, v = (rnd(batch, heads, seq, d) for _ in range(3))
     score = torch.empty(batch, heads, seq, seq, device="cuda", dtype=tdt)
-    ctx, out, inter = torch.empty(T, H, device="cuda", dtype=tdt), torch.empty(T, H, device="cuda", dtype=tdt), rnd(T, F)
+    ctx, out, inter = rnd(T, H), torch.empty(T, H, device="cuda", dtype=tdt), rnd(T, F)
     mask = torch.zeros(batch, seq, device="cuda")
 
     def fused(a, w, c, m, n, kk, epi, **kw):
@@ -160,6 +173,13 @@ def kernel_rooflines(dtype="f16", batch=64, seq=512, hidden=768, heads=12, ffn=3
         return lambda: capi.check(lib.ttmi_gemm_fused(P(a), P(w), P(c) if c is not None else None, m, n, kk, kk, kk, n, epi,
                                                       ctypes.byref(args), cdt, S()))
 
+    if only is not None:
+        # Counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): one copy of known size through
+        # ttmi_convert (fp32 -> fp32) to calibrate the counters' unit, then `iters` launches of the one kernel.
+        src = torch.zeros(COPY_ELEMS, device="cuda")
+        dst = torch.empty_like(src)
+        capi.check(lib.ttmi_convert(P(src), capi.F32, P(dst), capi.F32, COPY_ELEMS, S()))
+        torch.cuda.synchronize()
     res = {}
     gemms = {
         "qkv_gemm+bias+split": (fused(x, w_qkv, None, T, 3 * H, H, capi.EPI_QKV_SPLIT, bias=b_qkv, q=q, k=k, v=v, seq=seq,
@@ -179,6 +199,16 @@ def kernel_rooflines(dtype="f16", batch=64, seq=512, hidden=768, heads=12, ffn=3
     vt = torch.empty(batch, heads, d, seq, device="cuda", dtype=tdt).normal_()  # V kept transposed, as the layers do
     gemms["fused_attention"] = (lambda: capi.check(lib.ttmi_fused_attention(
         P(q), P(k), P(vt), P(mask), P(ctx), None, batch, heads, seq, d, seq, 0.125, cdt, S())), 4 * T * seq * H)
+    if only is not None:
+        membound_fns = {
+            "add_bias_layer_norm": lambda: capi.check(lib.ttmi_add_bias_layer_norm(
+                P(out), P(x), P(b_h), P(gam), P(b_h), T, H, 1e-12, cdt, S())),
+        }
+        fn = gemms[only][0] if only in gemms else membound_fns[only]
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return None
     for name, (fn, flops) in gemms.items():
         us = timed(fn)
         res[name] = {"bound": "mfma", "us": us, "achieved": flops / us / 1e6, "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
@@ -243,6 +273,9 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the other shapes of the metric")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline pass")
+    ap.add_argument("--pmc-kernel", default=None,
+                    help="counter-collection helper: run one calibration copy and a few launches of the named kernel "
+                         "of the roofline pass (e.g. ffn1_gemm+bias+gelu), print nothing, exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (requests are independent; there is no multi-GPU step to time); "
@@ -253,8 +286,11 @@ def main():
         sys.exit("bench.py: no GPU visible")
     import turbo_transformers  # noqa: F401  (fails loudly if the native libraries are missing)
 
-    head = run_dense(args.workload, args.steps, args.warmup)
     layers, hidden, heads, ffn, dtype, batch, seq = WORKLOADS[args.workload]
+    if args.pmc_kernel:
+        kernel_rooflines(dtype, batch, seq, hidden, heads, ffn, iters=3, only=args.pmc_kernel)
+        return
+    head = run_dense(args.workload, args.steps, args.warmup)
     line = {
         "metric": "bert_base_sequences_per_second", "value": head["seq_per_s"], "unit": "seq/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "p50_latency_ms": head["p50_ms"],
@@ -272,6 +308,11 @@ def main():
         r = kr[dom]
         line["roofline"] = {"kernel": dom, "bound": r["bound"], "achieved": r["achieved"], "peak": r["peak"], "unit": r["unit"],
                             "frac": r["frac"], "traffic": None, "avg_launch_us": r["us"]}
+        t = MEASURED_TRAFFIC.get((dom, dtype, batch, seq))
+        if t is not None:
+            line["roofline"]["traffic"] = t["fetch_bytes"] + t["write_bytes"]
+            line["roofline"]["traffic_detail"] = dict(t, unit="bytes per launch", algorithmic_bytes=2 * (
+                batch * seq * hidden + hidden * ffn + batch * seq * ffn))
         line["kernel_rooflines"] = {k: {"bound": v["bound"], "us": round(v["us"], 1), "achieved": round(v["achieved"], 1),
                                         "unit": v["unit"], "frac": round(v["frac"], 4),
                                         "launches_per_layer": v["launches_per_layer"]} for k, v in kr.items()}

@@ -83,6 +83,10 @@ constexpr int kD = 64;          // head dim
 constexpr int kBQ = 128;        // queries per workgroup
 constexpr int kBKV = 64;        // keys per LDS tile
 constexpr float kNegBig = -1.0e30f;
+// log2 of the largest probability tolerated before the running maximum is moved.  bf16 keeps the
+// exact maximum: with 8 mantissa bits a dominant probability of exactly 1.0 is worth keeping exact.
+template <typename T>
+constexpr float kSlack = sizeof(T) == 2 && !std::is_same<T, bf16>::value ? 8.0f : 0.0f;
 
 // Position of a key inside its group of 16 in an LDS V^T row.  A lane of the P.V MFMA holds the
 // probabilities of keys {4h..4h+3, 8+4h..8+4h+3} (h = lane/32) of the group; storing the group as
@@ -244,10 +248,21 @@ __global__ __launch_bounds__(256, 2) void fused_attention_kernel(const T* __rest
 #pragma unroll
       for (int e = 1; e < 16; ++e) mx = fmaxf(mx, st[e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
-      const float neg_m = -m_new * scale_log2e;
-      m_run = m_new;
+      // Lazy running maximum: the reference point m_run only moves when some query of the
+      // wavefront would otherwise see exp2 arguments above kSlack (fp16: probabilities up to 2^kSlack are
+      // as precise as smaller ones and the final division by the row sum cancels the choice of
+      // m_run), so the rescaling of the 32 output accumulators is skipped for most tiles.
+      if (__any((mx - m_run) * scale_log2e > kSlack<T>)) {
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) ot[t][e] *= alpha;
+      }
+      const float neg_m = -m_run * scale_log2e;
       Chunk16 pf[2];
       float psum = 0.f;
 #pragma unroll
@@ -258,13 +273,7 @@ __global__ __launch_bounds__(256, 2) void fused_attention_kernel(const T* __rest
         pf[w >> 2].w[w & 3] = pk;
         psum = add_pair<T>(pk, psum);
       }
-      l_run = l_run * alpha + psum;
-      if (__any(alpha != 1.0f)) {  // the running maximum rarely moves after the first tiles
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) ot[t][e] *= alpha;
-      }
+      l_run += psum;
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk)
 #pragma unroll

@@ -103,6 +103,19 @@ struct FastDiv {
   __device__ __forceinline__ uint32_t div(uint32_t n) const { return d == 1 ? n : (__umulhi(n, mul) >> shr); }
 };
 
+// Tile index -> (tile row, tile column), walking bands of kBandRows tile rows column by column, so
+// that the ~32 workgroups running side by side on one XCD cover a block of about 4 x 8 tiles and
+// share 4 A row-panels and 8 B column-panels in that XCD's L2 (row-major order would share one A
+// panel and stream 32 different B panels).
+constexpr int kBandRows = 4;
+__device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+  const int band = t / (kBandRows * tiles_n);
+  const int idx = t - band * (kBandRows * tiles_n);
+  const int rows = min(kBandRows, tiles_m - band * kBandRows);
+  tile_n = idx / rows;
+  tile_m = band * kBandRows + (idx - tile_n * rows);
+}
+
 struct GemmArgs {
   const char* a;
   const char* b;
@@ -422,7 +435,8 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
   const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
   const int logical = (int)(blockIdx.x % kNumXcd) * per_xcd + (int)(blockIdx.x / kNumXcd);
   if (logical >= tiles) return;
-  const int tile_m = logical / g.tiles_n, tile_n = logical % g.tiles_n;
+  int tile_m, tile_n;
+  tile_coords(logical, g.tiles_m, g.tiles_n, tile_m, tile_n);
   const int z = blockIdx.z;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
@@ -633,7 +647,9 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   const T* pa[A_LOADS];
   const T* pb[B_LOADS];
   auto point_at = [&](int tile) {
-    const int m0 = (tile / g.tiles_n) * BM, n0 = (tile % g.tiles_n) * BN;
+    int tile_m, tile_n;
+    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int sub = lane >> 3, p = lane & 7;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
@@ -710,7 +726,9 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   point_at(logical);
   issue(0);
   for (;;) {
-    const int m0 = (logical / g.tiles_n) * BM, n0 = (logical % g.tiles_n) * BN;
+    int tile_m, tile_n;
+    tile_coords(logical, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
     float bj[TN];
     load_bias_columns<TN>(epi, n0 + wn0 + lrow, g.n, bj);
 #pragma unroll

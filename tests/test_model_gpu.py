@@ -402,3 +402,44 @@ def test_quantized_bert_model_runs_and_tracks_fp32(tt):
     seq, pooled = qmodel(ids)[:2]
     assert seq.shape == (20, 128, cfg.hidden_size) and pooled.shape == (20, cfg.hidden_size)
     assert float((seq - want).abs().mean()) < 0.03  # int8 noise through 12 layers, not a parity bound
+
+
+def test_model_aware_schema_gives_the_same_forward(tt):
+    """python/tests/bert_model_test.py:64-105 with use_memory_opt: plan the activations for the input
+    shape, run under the "model-aware" schema, compare with the "naive" run of the same model.  The
+    plan changes between inputs (2x50 -> 4x16 -> 1x100 -> 2x50), the chunks are reused, and no planned
+    activation reaches the caching allocator."""
+    model, cfg = _hf_bert(3, seed=5)
+    tmodel = tt.BertModel.from_torch(model, torch.device("cuda:0"), "turbo")
+    cxx = tt.cxx
+    g = torch.Generator().manual_seed(3)
+    inputs = [torch.randint(0, cfg.vocab_size, shape, generator=g).cuda() for shape in [(2, 50), (4, 16), (1, 100), (2, 50)]]
+    naive = [tuple(t.clone() for t in tmodel(ids)[:2]) for ids in inputs]
+    torch.cuda.synchronize()
+    try:
+        tt.reset_allocator_schema("model-aware")
+        chunks_seen = []
+        for ids, want in zip(inputs, naive):
+            tt.bert_opt_mem_allocate_api(ids.shape[0], ids.shape[1], cfg.num_attention_heads, cfg.hidden_size,
+                                         cfg.num_hidden_layers, "GPU")
+            before = cxx.allocator_stats()
+            seq, pooled = tmodel(ids)[:2]
+            torch.cuda.synchronize()
+            assert torch.equal(seq, want[0]) and torch.equal(pooled, want[1])
+            chunks_seen.append(cxx.model_aware_chunks())
+            after = cxx.allocator_stats()
+            # second forward of the same shape: steady state, nothing new from the device
+            seq2 = tmodel(ids)[0]
+            torch.cuda.synchronize()
+            assert torch.equal(seq2, want[0])
+            assert cxx.allocator_stats()["device_mallocs"] == after["device_mallocs"]
+        assert all(n >= 1 and b >= (2 << 20) for n, b in chunks_seen)
+        # an input larger than the plan is refused with a message that says what to do
+        big = torch.randint(0, cfg.vocab_size, (4, 128), generator=g).cuda()
+        with pytest.raises(RuntimeError, match="bert_opt_mem_allocate_api"):
+            tmodel(big)
+    finally:
+        tt.reset_allocator_schema("naive")
+    seq = tmodel(inputs[0])[0]
+    torch.cuda.synchronize()
+    assert torch.equal(seq, naive[0][0])

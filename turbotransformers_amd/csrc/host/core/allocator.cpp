@@ -14,6 +14,19 @@ Allocator& Allocator::GetInstance() {
   return a;
 }
 
+// Chunks of the model-aware plan come straight from the device (they are few, large and long-lived)
+// and are returned only after the device has drained, since kernels may still be using them.
+Allocator::Allocator()
+    : plan_(new ModelAwarePlan(
+          [](size_t bytes) -> void* {
+            void* p = nullptr;
+            return ttmi_malloc(&p, bytes) == 0 ? p : nullptr;
+          },
+          [](void* p) {
+            ttmi_stream_sync(nullptr);
+            ttmi_free(p);
+          })) {}
+
 size_t Allocator::RoundSize(size_t size) {
   if (size == 0) size = 1;
   constexpr size_t kSmall = 512, kLarge = 2u << 20, kThreshold = 1u << 20;
@@ -31,6 +44,14 @@ void* Allocator::DeviceMalloc(size_t bytes) {
 }
 
 void* Allocator::allocate(size_t size, DLDeviceType dev, const std::string& name) {
+  if (IsGpu(dev) && is_activation(name)) {
+    std::lock_guard<std::mutex> g(mutex_);
+    return plan_->Address(name, size);
+  }
+  return NaiveAllocate(size, dev, name);
+}
+
+void* Allocator::NaiveAllocate(size_t size, DLDeviceType dev, const std::string& name) {
   if (dev == kDLCPU) {
     void* p = nullptr;
     if (posix_memalign(&p, 64, size == 0 ? 64 : size) != 0) throw BadAlloc("posix_memalign failed for " + name);
@@ -76,7 +97,7 @@ void Allocator::free(void* mem, DLDeviceType dev, const std::string&) {
   }
   std::lock_guard<std::mutex> g(mutex_);
   auto it = live_blocks_.find(mem);
-  TT_ENFORCE(it != live_blocks_.end(), "free of a pointer this allocator does not own");
+  TT_ENFORCE(it != live_blocks_.end(), "free of a pointer this allocator does not own (planned activations are never freed)");
   const size_t sz = it->second;
   live_blocks_.erase(it);
   free_blocks_.emplace(sz, mem);
@@ -102,21 +123,35 @@ AllocatorStats Allocator::stats() {
 }
 
 void Allocator::set_schema(const std::string& schema) {
-  // allocator_api.cpp:28-36 accepts "naive" and "model-aware"; the offline chunk planner of
-  // the latter is not part of this build, so only "naive" is accepted.
-  if (schema == "naive") {
-    schema_ = schema;
-    return;
-  }
-  if (schema == "model-aware") TT_THROW("allocator schema 'model-aware' is not built; use 'naive'");
-  TT_THROW("no schema called %s", schema.c_str());
+  // allocator_api.cpp:64-81: "naive" and "model-aware" are the registered schemas
+  TT_ENFORCE(schema == "naive" || schema == "model-aware", "no schema called %s", schema.c_str());
+  std::lock_guard<std::mutex> g(mutex_);
+  schema_ = schema;
+}
+
+bool Allocator::is_activation(const std::string& name) {
+  std::lock_guard<std::mutex> g(mutex_);
+  return schema_ == "model-aware" && plan_->Has(name);
+}
+
+void Allocator::set_config(int64_t batch_size, int64_t seq_len, int64_t num_head, int64_t hidden_size, int64_t num_layer) {
+  std::lock_guard<std::mutex> g(mutex_);
+  plan_->Reset(batch_size, seq_len, num_head, hidden_size, num_layer);
+}
+
+std::pair<size_t, int64_t> Allocator::model_aware_chunks() {
+  std::lock_guard<std::mutex> g(mutex_);
+  return {plan_->chunk_count(), plan_->chunk_bytes()};
 }
 
 void reset_allocator_schema(const std::string& name) { Allocator::GetInstance().set_schema(name); }
 
-void bert_opt_mem_allocate_api(int64_t, int64_t, int64_t, int64_t, int64_t, const std::string&) {
-  // Only meaningful for the model-aware schema (allocator_api.cpp:112-125): a no-op under "naive".
-  TT_ENFORCE(Allocator::GetInstance().schema() == "naive", "unexpected allocator schema");
+void bert_opt_mem_allocate_api(int64_t batch_size, int64_t seq_len, int64_t num_head, int64_t hidden_size, int64_t num_layer,
+                               const std::string& dev_str) {
+  // allocator_api.cpp:112-118.  Only device activations are planned here; host tensors of this
+  // build are a few ids and always come from the heap.
+  TT_ENFORCE(dev_str == "GPU" || dev_str == "CPU", "device must be \"GPU\" or \"CPU\"");
+  if (dev_str == "GPU") Allocator::GetInstance().set_config(batch_size, seq_len, num_head, hidden_size, num_layer);
 }
 
 }  // namespace allocator

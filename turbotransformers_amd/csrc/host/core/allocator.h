@@ -10,16 +10,23 @@
 //            hipMalloc fails, every cached block is released and the request retried once
 //            (naive_allocator.h:50-63).  Reuse is ordered by the single work stream.
 //
+//   "model-aware"  device tensors whose name is one of the planned BERT activations live at a fixed
+//            offset of a few large chunks (core/model_aware_allocator.h), decided by
+//            bert_opt_mem_allocate_api(batch, seq, heads, hidden, layers, dev) before the forward;
+//            they are never freed individually.  Everything else goes the "naive" way.
+//
 // With 288 GB of HBM per GPU the cache is never trimmed on its own; FreeAllCached() does it.
 #pragma once
 
 #include <cstddef>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <unordered_map>
 
 #include "core/dlpack.h"
+#include "core/model_aware_allocator.h"
 
 namespace turbo_transformers {
 namespace core {
@@ -51,7 +58,13 @@ class Allocator {
 
   void set_schema(const std::string& schema);
   const std::string& schema() const { return schema_; }
-  bool is_activation(const std::string&) const { return false; }
+  // True when the model-aware schema is active and `name` is one of its planned activations:
+  // such memory is owned by the plan, not by the tensor that points at it.
+  bool is_activation(const std::string& name);
+  // Plan the activations of a BERT of this shape (allocator_api.cpp:83-88).
+  void set_config(int64_t batch_size, int64_t seq_len, int64_t num_head, int64_t hidden_size, int64_t num_layer);
+  // Chunks held by the model-aware plan (count, bytes).
+  std::pair<size_t, int64_t> model_aware_chunks();
 
   void FreeAllCached();
   AllocatorStats stats();
@@ -61,8 +74,10 @@ class Allocator {
   static size_t RoundSize(size_t size);
 
  private:
-  Allocator() = default;
+  Allocator();
+  ~Allocator() { plan_.release(); }  // chunks are left to process teardown: the device runtime may already be gone
   void* DeviceMalloc(size_t bytes);
+  void* NaiveAllocate(size_t size, DLDeviceType dev, const std::string& name);
 
   std::string schema_ = "naive";
   std::mutex mutex_;
@@ -71,6 +86,7 @@ class Allocator {
   AllocatorStats stats_;
   size_t device_limit_ = 0;
   size_t device_bytes_ = 0;
+  std::unique_ptr<ModelAwarePlan> plan_;
 };
 
 // Free functions with the reference's names (allocator_api.cpp:112-125).

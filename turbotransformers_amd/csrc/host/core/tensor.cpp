@@ -43,6 +43,10 @@ void OwnedDeleter(DLManagedTensor* self) {
   delete block;
 }
 
+// Memory placed by the model-aware plan belongs to the plan (tensor.cpp:46-53 of the reference:
+// DLManagedTensorDeletorWithoutData): only the descriptor is released.
+void PlannedDeleter(DLManagedTensor* self) { delete static_cast<OwnedBlock*>(self->manager_ctx); }
+
 int64_t Numel(const std::vector<int64_t>& shape) {
   return std::accumulate(shape.begin(), shape.end(), (int64_t)1, std::multiplies<int64_t>());
 }
@@ -59,8 +63,10 @@ DLManagedTensor* NewDLPackTensor(const std::vector<int64_t>& shape, DLDataType d
   block->name = name;
   block->capacity_bytes = (size_t)Numel(shape) * (dtype.bits / 8);
   DLTensor& t = block->managed.dl_tensor;
+  auto& alloc = allocator::Allocator::GetInstance();
+  const bool planned = IsGpu(device) && alloc.is_activation(name);
   try {
-    t.data = allocator::Allocator::GetInstance().allocate(block->capacity_bytes, device, name);
+    t.data = alloc.allocate(block->capacity_bytes, device, name);
   } catch (...) {
     delete block;
     throw;
@@ -74,7 +80,7 @@ DLManagedTensor* NewDLPackTensor(const std::vector<int64_t>& shape, DLDataType d
   t.strides = nullptr;
   t.byte_offset = 0;
   block->managed.manager_ctx = block;
-  block->managed.deleter = OwnedDeleter;
+  block->managed.deleter = planned ? PlannedDeleter : OwnedDeleter;
   return &block->managed;
 }
 
@@ -91,8 +97,11 @@ void* Tensor::ReshapeAs(DLDataType dtype, const std::vector<int64_t>& shape_list
   shadow_.reset();  // new contents: a producer that wants an fp32 copy calls EnsureShadow() afterwards
   const size_t need = (size_t)Numel(shape_list) * (dtype.bits / 8);
   // Reuse only buffers allocated here (their shape storage and capacity are ours); tensors
-  // imported from another framework are never resized in place.
-  if (managed_ != nullptr && managed_->deleter == OwnedDeleter) {
+  // imported from another framework are never resized in place.  A planned activation is looked up
+  // again on every call: the plan may have changed, and a planned address must not be kept once
+  // the schema is back to "naive".
+  const bool planned = IsGpu(device_type) && allocator::Allocator::GetInstance().is_activation(name);
+  if (!planned && managed_ != nullptr && managed_->deleter == OwnedDeleter) {
     auto* block = static_cast<OwnedBlock*>(managed_->manager_ctx);
     DLTensor& t = managed_->dl_tensor;
     const bool same_place = (IsGpu(t.device.device_type) == IsGpu(device_type)) &&

@@ -262,6 +262,36 @@ PYBIND11_MODULE(turbo_transformers_cxx, m) {
     d["oom_retries"] = s.oom_retries;
     return d;
   });
+  m.def("allocator_schema", [] { return core::allocator::Allocator::GetInstance().schema(); });
+  m.def("model_aware_chunks", [] { return core::allocator::Allocator::GetInstance().model_aware_chunks(); },
+        "(number of chunks, total bytes) held by the model-aware plan");
+  // The planner as plain functions, for tests: records are (name, start_op, end_op, size).
+  using Rec = std::tuple<std::string, int64_t, int64_t, int64_t>;
+  auto to_records = [](const std::vector<Rec>& in) {
+    std::vector<core::allocator::TensorRecord> out;
+    for (const auto& r : in) out.push_back({std::get<0>(r), std::get<1>(r), std::get<2>(r), std::get<3>(r)});
+    return out;
+  };
+  m.def("bert_tensor_usage_records", [](int64_t b, int64_t s, int64_t h, int64_t hidden, int64_t layers) {
+    std::vector<Rec> out;
+    for (const auto& r : core::allocator::BertTensorUsageRecords(b, s, h, hidden, layers))
+      out.emplace_back(r.name, r.start_op, r.end_op, r.size);
+    return out;
+  });
+  m.def("plan_memory", [to_records](const std::vector<Rec>& records, std::vector<int64_t> chunk_sizes) {
+    std::vector<core::allocator::Placement> placements;
+    std::vector<bool> used;
+    core::allocator::ChunkedGreedyBySizeOffsetCalculation(to_records(records), &chunk_sizes, &placements, &used);
+    std::vector<std::pair<int, int64_t>> pl;
+    for (const auto& p : placements) pl.emplace_back(p.chunk, p.offset);
+    return py::make_tuple(pl, chunk_sizes, used);
+  }, "-> (placements [(chunk, offset)], chunk sizes, chunk used flags)");
+  m.def("placement_is_valid", [to_records](const std::vector<Rec>& records, const std::vector<int64_t>& chunk_sizes,
+                                           const std::vector<std::pair<int, int64_t>>& placements) {
+    std::vector<core::allocator::Placement> pl;
+    for (const auto& p : placements) pl.push_back({p.first, p.second});
+    return core::allocator::PlacementIsValid(to_records(records), chunk_sizes, pl);
+  });
   m.def("set_allocator_device_limit_for_test",
         [](size_t bytes) { core::allocator::Allocator::GetInstance().set_device_limit_for_test(bytes); });
   m.def("load_npz",

@@ -208,6 +208,13 @@ TTMI_API int ttmi_smart_pad_mask(float* mask, const int32_t* cu_seqlens, int64_t
  * keep every weight K-contiguous ([out,in]) for the MFMA kernels. */
 TTMI_API int ttmi_transpose_2d(const void* in, void* out, int64_t rows, int64_t cols, int dtype, void* stream);
 
+/* kernels::Concat<T>  (layers/kernels/utils.cpp:33-93), the decoder's key/value cache append:
+ * out[o, 0:a_inner] = a[o, :], out[o, a_inner:] = b[o, :] for o < outer, i.e. a concatenation along
+ * one dimension with outer = product of the dimensions before it and *_inner = that dimension's
+ * size times the product of the dimensions after it.  Pure data movement, any dtype. */
+TTMI_API int ttmi_concat(const void* a, const void* b, void* out, int64_t outer, int64_t a_inner, int64_t b_inner,
+                         int dtype, void* stream);
+
 /* Element type conversion between TTMI_F32 / F16 / BF16 buffers. */
 TTMI_API int ttmi_convert(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, void* stream);
 
@@ -261,7 +268,9 @@ typedef struct ttmi_epilogue_args {
   void* q; void* k; void* v; /* outputs [B,h,S,d]                   (QKV_SPLIT[_PAD])        */
   int64_t seq;               /* S (or max_seq for the padded form)                          */
   int64_t heads;             /* h                                                           */
-  int64_t head_dim;          /* d; N must equal 3*h*d                                       */
+  int64_t head_dim;          /* d; N must equal 3*h*d, or h*d: then only q is written -- MatMul +
+                                AddBiasTransposeForScore of one projection
+                                (layers/multi_headed_attention.cpp:73-88)                   */
   const int32_t* token_rows; /* device [M]: packed token -> b*max_seq+s (QKV_SPLIT_PAD)      */
   int64_t batch;             /* B                                   (QKV_SPLIT_PAD)          */
   int64_t v_seq_pitch;       /* 0: v is [B,h,S,d]; > 0: v is written transposed as

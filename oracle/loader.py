@@ -230,6 +230,79 @@ class Oracle:
                                         _fp(out), _fp(attn))
         return out, attn
 
+    @staticmethod
+    def concat(a, b, dim):
+        """kernels::Concat<float> (layers/kernels/utils.cpp:33-93): rows of `a` then rows of `b` along
+        `dim`; data movement only, so NumPy's routine is the restatement."""
+        return np.ascontiguousarray(np.concatenate([a, b], axis=dim), np.float32)
+
+    def add_bias_transpose_for_score(self, x, bias, B, S, h, d):
+        """kernels::AddBiasTransposeForScore (layers/kernels/transpose.cpp:194-232): [B,S,h,d] + bias[h*d]
+        -> [B,h,S,d].  It is the one-output case of the split kernel, restated through it with two dummy
+        thirds so that the arithmetic (one fp32 add) is the oracle's own."""
+        x3 = np.zeros((B * S, 3, h * d), np.float32)
+        x3[:, 0, :] = np.asarray(x, np.float32).reshape(B * S, h * d)
+        b3 = np.concatenate([np.asarray(bias, np.float32), np.zeros(2 * h * d, np.float32)])
+        return self.split_add_bias_transpose(x3.reshape(B * S, 3 * h * d), b3, B, S, h, d)[0]
+
+    def multi_headed_attention(self, key, value, query, mask, w, heads, attn_type="self", layer_cache=None,
+                               pre_layernorm=False, post_layernorm=False, post_add_input=False):
+        """layers::MultiHeadedAttention::operator() (layers/multi_headed_attention.cpp:260-380) with both
+        projections paths (:35-164 context, :168-232 self), composed from the oracle's kernels.
+
+        w: dict with q_w,k_w,v_w [H,H] ([in,out]), q_b,k_b,v_b, qkv_w [H,3H], qkv_b, dense_w, dense_b and,
+        when a LayerNorm is used, ln_g, ln_b.  layer_cache: dict of float32 arrays or None entries
+        (self_keys/self_values/memory_keys/memory_values); it is updated in place like the reference's.
+        mask: additive fp32, (B,1,T) or (B,F,T), or None.  Returns (output [B,F,H], attn [B,h,F,T])."""
+        f32 = lambda a: np.ascontiguousarray(a, np.float32)
+        query = f32(query)
+        B, F, H = query.shape
+        d = H // heads
+        cache = layer_cache if layer_cache is not None else {}
+        has = lambda name: cache.get(name) is not None
+        q_in = query
+        if pre_layernorm:  # :66-80 / :190-199, eps hard-coded 1e-6
+            q_in = self.layer_norm(query, w["ln_g"], w["ln_b"], 1e-6)
+        if attn_type == "self":
+            qkv = self.matmul(q_in.reshape(B * F, H), f32(w["qkv_w"]))
+            q, k, v = self.split_add_bias_transpose(qkv, f32(w["qkv_b"]), B, F, heads, d)
+            if has("self_keys"):
+                k = self.concat(f32(cache["self_keys"]), k, 2)
+            if has("self_values"):
+                v = self.concat(f32(cache["self_values"]), v, 2)
+            if layer_cache:  # non-empty dict: the grown keys/values go back into the cache (:216-229)
+                cache["self_keys"], cache["self_values"] = k.copy(), v.copy()
+        elif attn_type == "context":
+            q = self.add_bias_transpose_for_score(self.matmul(q_in.reshape(B * F, H), f32(w["q_w"])), w["q_b"], B, F, heads, d)
+            if has("memory_keys") and has("memory_values"):
+                k, v = f32(cache["memory_keys"]), f32(cache["memory_values"])
+            else:
+                key, value = f32(key), f32(value)
+                Tk = key.shape[1]
+                k = self.add_bias_transpose_for_score(self.matmul(key.reshape(B * Tk, H), f32(w["k_w"])), w["k_b"], B, Tk, heads, d)
+                v = self.add_bias_transpose_for_score(self.matmul(value.reshape(B * Tk, H), f32(w["v_w"])), w["v_b"], B, Tk, heads, d)
+                if layer_cache:
+                    cache["memory_keys"], cache["memory_values"] = k.copy(), v.copy()
+        else:
+            raise ValueError("attn_type should be context or self.")
+        T = k.shape[2]
+        score = self.batch_matmul(q, k, True, 1.0 / np.sqrt(np.float32(d)))
+        is_2d = True
+        m = None
+        if mask is not None:
+            m = f32(mask)
+            is_2d = m.size == B * T
+        attn = self.apply_mask_and_softmax(score, m, 1.0, is_2d)
+        ctx = self.transpose_for_score(self.batch_matmul(attn, v, False)).reshape(B * F, H)
+        out = self.matmul(ctx, f32(w["dense_w"])).reshape(B, F, H)
+        if post_add_input:       # AddInputBias (:371-373)
+            out = out + query + f32(w["dense_b"])
+        elif post_layernorm:     # AddBiasLayerNorm with the query as residual, eps 1e-12 (:363-369)
+            out = self.add_bias_layer_norm(out, query, f32(w["dense_b"]), f32(w["ln_g"]), f32(w["ln_b"]), 1e-12)
+        else:                    # AddBias (:360-361)
+            out = out + f32(w["dense_b"])
+        return f32(out), attn
+
     def bert_layer(self, x, mask, w, heads):
         B, S, H = x.shape
         F = w["inter_w"].shape[1]

@@ -180,6 +180,26 @@ def test_fused_qkv_split(ttmi, oracle, dt, B, S, h, d, v_transposed):
 
 
 @pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("B,S,h,d", [(2, 11, 4, 64), (3, 128, 12, 64), (2, 5, 3, 20)])
+def test_fused_single_projection_to_heads(ttmi, oracle, dt, B, S, h, d):
+    """MatMul + AddBiasTransposeForScore of one projection (context attention, multi_headed_attention.cpp:73-88)
+    as the one-output case of the QKV epilogue: N = h*d, only q is written."""
+    import ctypes
+    rng = np.random.default_rng(S * 7)
+    H = h * d
+    A, W = _ab(rng, B * S, H, H, 1)
+    bias = rng.standard_normal(H).astype(np.float32)
+    dA, dW, db = dev(A, dt), dev(W, dt), dev(bias, dt)
+    q = torch.empty((B, h, S, d), dtype=dA.dtype, device="cuda")
+    args = _epi(bias=db, q=q, seq=S, heads=h, head_dim=d)
+    ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), None, B * S, H, H, H, H, H, capi.EPI_QKV_SPLIT, ctypes.byref(args),
+                            TTMI_DTYPES[dt], stream()))
+    proj = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    want = oracle.add_bias_transpose_for_score(proj, rounded(bias, dt), B, S, h, d)
+    assert max_abs(host(q), want) <= GEMM_TOL[dt] * 2
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
 @pytest.mark.parametrize("v_transposed", [False, True])
 @pytest.mark.parametrize("lens", [[9, 30, 1, 17], [64, 8, 200, 16, 33]])
 def test_fused_qkv_split_pad(ttmi, oracle, dt, lens, v_transposed):

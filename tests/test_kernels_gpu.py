@@ -269,6 +269,23 @@ def test_transpose_2d_and_convert(ttmi, dt):
     assert np.array_equal(host(f), rounded(x, dt))
 
 
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("shape_a,shape_b,dim", [((2, 3, 5, 8), (2, 3, 1, 8), 2), ((4, 7), (4, 9), 1), ((3, 5, 6), (2, 5, 6), 0),
+                                               ((2, 2, 3, 5), (2, 2, 4, 5), 2), ((6, 0, 4), (6, 3, 4), 1)])
+def test_concat(ttmi, oracle, dt, shape_a, shape_b, dim):
+    """kernels::Concat (utils.cpp:33-93): bit-exact data movement, every alignment path (16/4/2-byte units)."""
+    rng = np.random.default_rng(sum(shape_a))
+    a, b = rng.standard_normal(shape_a, np.float32), rng.standard_normal(shape_b, np.float32)
+    want = oracle.concat(rounded(a, dt), rounded(b, dt), dim)
+    da, db = dev(a, dt), dev(b, dt)
+    out = torch.full(want.shape, 5.0, dtype=da.dtype, device="cuda")
+    outer = int(np.prod(shape_a[:dim]))
+    inner = lambda sh: int(np.prod(sh[dim:]))
+    ok(ttmi.ttmi_concat(ptr(da) if a.size else None, ptr(db), ptr(out), outer, inner(shape_a), inner(shape_b), TTMI_DTYPES[dt],
+                        stream()))
+    assert np.array_equal(host(out), want)
+
+
 def test_memcpy_and_memset(ttmi):
     a = np.arange(1000, dtype=np.float32)
     d = torch.empty(1000, device="cuda")

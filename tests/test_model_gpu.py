@@ -443,3 +443,154 @@ def test_model_aware_schema_gives_the_same_forward(tt):
     seq = tmodel(inputs[0])[0]
     torch.cuda.synchronize()
     assert torch.equal(seq, naive[0][0])
+
+
+# ---------------------------------------------------------------- general MultiHeadedAttention
+class _OnmtLikeAttention(torch.nn.Module):
+    """A module with OpenNMT-py's MultiHeadedAttention parameter names (onmt/modules/multi_headed_attn.py);
+    OpenNMT itself is not installed, so the comparator below restates its forward with torch routines."""
+
+    def __init__(self, heads, hidden):
+        super().__init__()
+        self.head_count, self.max_relative_positions = heads, 0
+        self.linear_keys = torch.nn.Linear(hidden, hidden)
+        self.linear_values = torch.nn.Linear(hidden, hidden)
+        self.linear_query = torch.nn.Linear(hidden, hidden)
+        self.final_linear = torch.nn.Linear(hidden, hidden)
+
+
+def _mha_weights(mod, ln=None):
+    t = lambda p: p.detach().cpu().numpy().T.copy()
+    v = lambda p: p.detach().cpu().numpy().copy()
+    w = {"q_w": t(mod.linear_query.weight), "k_w": t(mod.linear_keys.weight), "v_w": t(mod.linear_values.weight),
+         "q_b": v(mod.linear_query.bias), "k_b": v(mod.linear_keys.bias), "v_b": v(mod.linear_values.bias),
+         "dense_w": t(mod.final_linear.weight), "dense_b": v(mod.final_linear.bias)}
+    w["qkv_w"] = np.concatenate([w["q_w"], w["k_w"], w["v_w"]], 1)
+    w["qkv_b"] = np.concatenate([w["q_b"], w["k_b"], w["v_b"]])
+    if ln is not None:
+        w["ln_g"], w["ln_b"] = v(ln.weight), v(ln.bias)
+    return w
+
+
+def _torch_attention(mod, key, value, query, mask):
+    """softmax(q k^T / sqrt(d) + mask) v through torch's own fused routine, then the final projection."""
+    B, F, H = query.shape
+    h = mod.head_count
+    heads = lambda x: x.view(B, -1, h, H // h).transpose(1, 2)
+    q, k, v = heads(mod.linear_query(query)), heads(mod.linear_keys(key)), heads(mod.linear_values(value))
+    m = None if mask is None else mask.view(B, 1, mask.shape[-2], mask.shape[-1])
+    ctx = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=m)
+    return mod.final_linear(ctx.transpose(1, 2).reshape(B, F, H))
+
+
+def _make_mha(tt, heads=4, hidden=256, seed=0, dtype=torch.float32):
+    torch.manual_seed(seed)
+    mod = _OnmtLikeAttention(heads, hidden).cuda().to(dtype).eval()
+    ln = torch.nn.LayerNorm(hidden, eps=1e-6).cuda().to(dtype)
+    with torch.no_grad():
+        ln.weight.add_(0.1 * torch.randn_like(ln.weight))
+        ln.bias.add_(0.1 * torch.randn_like(ln.bias))
+    return mod, ln, tt.MultiHeadedAttention.from_onmt(mod, ln)
+
+
+@pytest.mark.parametrize("attn_type", ["self", "context"])
+@pytest.mark.parametrize("variant", ["bias", "post_layernorm", "post_add_input", "pre_layernorm+add"])
+def test_multi_headed_attention_variants(tt, oracle, attn_type, variant):
+    """layers/multi_headed_attention.cpp:260-380: both projection paths and every output form, against the
+    oracle's composition; the plain form also against torch's scaled_dot_product_attention."""
+    B, F, T, H, h = 3, 7, (7 if attn_type == "self" else 11), 256, 4
+    mod, ln, layer = _make_mha(tt, h, H, seed=F + T)
+    g = torch.Generator().manual_seed(1)
+    query = torch.randn(B, F, H, generator=g).cuda()
+    memory = query if attn_type == "self" else torch.randn(B, T, H, generator=g).cuda()
+    mask = torch.zeros(B, 1, T)
+    mask[0, 0, T - 3:] = -1e9
+    mask[2, 0, :2] = -1e9
+    mask = mask.cuda()
+    kw = {"bias": {}, "post_layernorm": {"post_layernorm": True}, "post_add_input": {"post_add_input": True},
+          "pre_layernorm+add": {"pre_layernorm": True, "post_add_input": True}}[variant]
+    out, attn = layer(memory, memory, query, mask=mask, layer_cache=None, attn_type=attn_type, **kw)
+    want_out, want_attn = oracle.multi_headed_attention(host(memory), host(memory), host(query), host(mask), _mha_weights(mod, ln),
+                                                        h, attn_type, None, **kw)
+    assert tuple(attn.shape) == (B, h, F, T)
+    assert max_abs(host(attn), want_attn) < 1e-5
+    assert max_abs(host(out), want_out) < 2e-4
+    if variant == "bias":
+        with torch.no_grad():
+            ref = _torch_attention(mod, memory, memory, query, mask)
+        assert max_abs(host(out), host(ref)) < 2e-4
+        assert np.allclose(host(attn).sum(-1), 1.0, atol=1e-5) and host(attn)[0, :, :, T - 3:].max() == 0.0
+
+
+def test_multi_headed_attention_self_cache_equals_full_causal_attention(tt, oracle):
+    """Decoder self attention one position at a time with a growing self_keys/self_values cache
+    (:205-229) must reproduce full attention under a causal mask, and the cache must hold all keys."""
+    B, S, H, h = 2, 6, 256, 4
+    mod, ln, layer = _make_mha(tt, h, H, seed=3)
+    x = torch.randn(B, S, H, generator=torch.Generator().manual_seed(2)).cuda()
+    causal = torch.triu(torch.full((S, S), -1e9), diagonal=1).expand(B, S, S).contiguous().cuda()
+    full, _ = layer(x, x, x, mask=causal, layer_cache=None, attn_type="self", post_layernorm=True)
+    cache = {"self_keys": None, "self_values": None, "memory_keys": None, "memory_values": None}
+    ocache = dict(cache)
+    w = _mha_weights(mod, ln)
+    for t in range(S):
+        step = x[:, t:t + 1].contiguous()
+        out, attn = layer(step, step, step, mask=None, layer_cache=cache, attn_type="self", post_layernorm=True)
+        want, _ = oracle.multi_headed_attention(host(step), host(step), host(step), None, w, h, "self", ocache, post_layernorm=True)
+        assert tuple(attn.shape) == (B, h, 1, t + 1)
+        assert tuple(cache["self_keys"].shape) == (B, h, t + 1, H // h) and cache["memory_keys"] is None
+        assert max_abs(host(out), want) < 2e-4
+        assert max_abs(host(out), host(full[:, t:t + 1])) < 2e-4
+        assert max_abs(host(cache["self_keys"]), ocache["self_keys"]) < 1e-5
+        assert max_abs(host(cache["self_values"]), ocache["self_values"]) < 1e-5
+
+
+def test_multi_headed_attention_context_memory_cache(tt, oracle):
+    """Context attention projects the encoder memory once (:107-150), keeps it in memory_keys/values and
+    reuses it on later calls (:90-105) -- even when different key/value tensors are passed then."""
+    B, F, T, H, h = 2, 3, 9, 256, 4
+    mod, ln, layer = _make_mha(tt, h, H, seed=4)
+    g = torch.Generator().manual_seed(5)
+    memory, q1, q2 = (torch.randn(B, n, H, generator=g).cuda() for n in (T, F, F))
+    mask = torch.zeros(B, 1, T)
+    mask[1, 0, 5:] = -1e18  # OpenNMT's fill value; must not produce NaN
+    mask = mask.cuda()
+    cache = {"memory_keys": None, "memory_values": None, "self_keys": None, "self_values": None}
+    out1, _ = layer(memory, memory, q1, mask=mask, layer_cache=cache, attn_type="context")
+    assert tuple(cache["memory_keys"].shape) == (B, h, T, H // h) and cache["self_keys"] is None
+    w = _mha_weights(mod, ln)
+    want1, _ = oracle.multi_headed_attention(host(memory), host(memory), host(q1), host(mask), w, h, "context", None)
+    assert max_abs(host(out1), want1) < 2e-4
+    keys = cache["memory_keys"].clone()
+    garbage = torch.full_like(memory, 7.0)
+    out2, _ = layer(garbage, garbage, q2, mask=mask, layer_cache=cache, attn_type="context")
+    want2, _ = oracle.multi_headed_attention(host(memory), host(memory), host(q2), host(mask), w, h, "context", None)
+    assert max_abs(host(out2), want2) < 2e-4
+    assert torch.equal(cache["memory_keys"], keys)
+    assert np.isfinite(host(out2)).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_multi_headed_attention_half_precision(tt, oracle, dtype):
+    B, F, T, H, h = 2, 16, 24, 256, 4
+    mod, ln, layer = _make_mha(tt, h, H, seed=6, dtype=dtype)
+    g = torch.Generator().manual_seed(7)
+    query, memory = torch.randn(B, F, H, generator=g).cuda().to(dtype), torch.randn(B, T, H, generator=g).cuda().to(dtype)
+    out, attn = layer(memory, memory, query, mask=None, layer_cache=None, attn_type="context", post_layernorm=True)
+    assert out.dtype == dtype
+    f = lambda t: host(t.float())
+    w = {k: v for k, v in _mha_weights(mod.float(), ln.float()).items()}
+    want, _ = oracle.multi_headed_attention(f(memory), f(memory), f(query), None, w, h, "context", None, post_layernorm=True)
+    assert max_abs(f(out), want) < (2e-2 if dtype == torch.float16 else 6e-2)
+
+
+def test_multi_headed_attention_rejects_bad_arguments(tt):
+    mod, ln, layer = _make_mha(tt, 4, 256)
+    x = torch.randn(2, 5, 256).cuda()
+    with pytest.raises(RuntimeError, match="context or self"):
+        layer(x, x, x, attn_type="cross")
+    with pytest.raises(RuntimeError, match="key and value"):
+        layer(x[:, :3].contiguous(), x, x, attn_type="context")
+    bad = {"self_keys": torch.zeros(2, 4, 3, 32).cuda(), "self_values": torch.zeros(2, 4, 3, 64).cuda()}
+    with pytest.raises(RuntimeError, match="layer_cache"):
+        layer(x, x, x, layer_cache=bad, attn_type="self")

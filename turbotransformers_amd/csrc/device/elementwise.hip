@@ -286,6 +286,20 @@ __global__ __launch_bounds__(256) void transpose_2d_kernel(const T* __restrict__
     if (c0 + j < cols && r0 + tx < rows) out[(c0 + j) * rows + r0 + tx] = tile[tx][j];
 }
 
+// out[o, :] = a[o, :] ++ b[o, :] for `outer` rows; U is the widest unit (16, 4, 2 or 1 bytes) that
+// divides both row lengths and all three base addresses.  Lengths are in units of U.
+template <typename U>
+__global__ __launch_bounds__(256) void concat_kernel(const U* __restrict__ a, const U* __restrict__ b, U* __restrict__ out,
+                                                     int64_t outer, int64_t a_len, int64_t b_len) {
+  const int64_t row_len = a_len + b_len, total = outer * row_len;
+  int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i < total; i += stride) {
+    const int64_t o = i / row_len, j = i - o * row_len;
+    out[i] = j < a_len ? a[o * a_len + j] : b[o * b_len + (j - a_len)];
+  }
+}
+
 template <typename S, typename D>
 __global__ void convert_kernel(const S* __restrict__ src, D* __restrict__ dst, int64_t n) {
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
@@ -522,6 +536,28 @@ int ttmi_transpose_2d(const void* in, void* out, int64_t rows, int64_t cols, int
     default: return fail(TTMI_EINVAL, "unsupported dtype for transpose_2d");
   }
   return launch_status("transpose_2d");
+}
+
+int ttmi_concat(const void* a, const void* b, void* out, int64_t outer, int64_t a_inner, int64_t b_inner, int dtype,
+                void* stream) {
+  TTMI_REQUIRE(out && (a || a_inner == 0) && (b || b_inner == 0), "null tensor");
+  TTMI_REQUIRE(outer >= 0 && a_inner >= 0 && b_inner >= 0, "negative size");
+  const int64_t esz = (int64_t)dtype_size(dtype);
+  TTMI_REQUIRE(esz > 0, "unsupported dtype for concat");
+  if (outer * (a_inner + b_inner) == 0) return 0;
+  const int64_t ab = a_inner * esz, bb = b_inner * esz;  // bytes per row
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(out) |
+                         (uintptr_t)ab | (uintptr_t)bb;
+  hipStream_t s = (hipStream_t)stream;
+#define TTMI_CONCAT_AS(U)                                                                                             \
+  hipLaunchKernelGGL((concat_kernel<U>), dim3(flat_grid(outer * (ab + bb) / (int64_t)sizeof(U))), dim3(256), 0, s,  \
+                     (const U*)a, (const U*)b, (U*)out, outer, ab / (int64_t)sizeof(U), bb / (int64_t)sizeof(U))
+  if ((bits & 15) == 0) TTMI_CONCAT_AS(uint4);
+  else if ((bits & 3) == 0) TTMI_CONCAT_AS(uint32_t);
+  else if ((bits & 1) == 0) TTMI_CONCAT_AS(uint16_t);
+  else TTMI_CONCAT_AS(uint8_t);
+#undef TTMI_CONCAT_AS
+  return launch_status("concat");
 }
 
 int ttmi_convert(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, void* stream) {

@@ -1013,9 +1013,11 @@ int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n,
       case TTMI_EPI_QKV_SPLIT:
       case TTMI_EPI_QKV_SPLIT_PAD: {
         const bool pad = epilogue == TTMI_EPI_QKV_SPLIT_PAD;
-        TTMI_REQUIRE(args->q && args->k && args->v && args->bias, "QKV epilogue needs q, k, v, bias");
         TTMI_REQUIRE(args->seq > 0 && args->heads > 0 && args->head_dim > 0, "QKV epilogue needs seq/heads/head_dim");
-        TTMI_REQUIRE(n == 3 * args->heads * args->head_dim, "N must be 3*heads*head_dim");
+        const bool single = n == args->heads * args->head_dim;  // one projection: only q is written
+        TTMI_REQUIRE(single || n == 3 * args->heads * args->head_dim, "N must be heads*head_dim or 3*heads*head_dim");
+        TTMI_REQUIRE(args->q && args->bias && (single || (args->k && args->v)), "QKV epilogue needs q, k, v, bias");
+        TTMI_REQUIRE(!single || args->v_seq_pitch == 0, "v_seq_pitch needs the three-way split");
         if (pad) TTMI_REQUIRE(args->token_rows != nullptr && args->batch > 0, "padded QKV epilogue needs token_rows and batch");
         else TTMI_REQUIRE(m % args->seq == 0, "M must be a multiple of seq");
         const int hidden = (int)(args->heads * args->head_dim);

@@ -46,10 +46,10 @@ bool MultiHeadedAttention::UseFusedCore(const Tensor& attention_mask, const Tens
 static int64_t RoundUp8(int64_t n) { return (n + 7) / 8 * 8; }
 
 // score -> softmax -> P V -> merge heads -> output projection -> bias (+input) (+LayerNorm)
-void MultiHeadedAttention::SelfAttentionTail(const Tensor& query_tensor, const Tensor& attention_mask, Tensor* output,
-                                             Tensor* att_score, int64_t batch, int64_t seq,
-                                             const std::vector<int64_t>* seq_list, int64_t v_pitch, bool post_layernorm,
-                                             bool post_add_input, bool is_trans_weight) const {
+void MultiHeadedAttention::AttentionTail(const Tensor& query_tensor, const Tensor& attention_mask, Tensor* output,
+                                         Tensor* att_score, int64_t batch, int64_t seq, int64_t key_seq, const Tensor& k,
+                                         const Tensor& v, const std::vector<int64_t>* seq_list, int64_t v_pitch,
+                                         bool post_layernorm, bool post_add_input, bool is_trans_weight) const {
   const int dt = kernels::DeviceDType(query_tensor);
   const DLDeviceType dev = query_tensor.device_type();
   const int dev_id = query_tensor.device_id();
@@ -67,28 +67,32 @@ void MultiHeadedAttention::SelfAttentionTail(const Tensor& query_tensor, const T
       TT_ENFORCE_EQ(attention_mask.numel(), batch * seq, "attention mask has the wrong size");
       mask = attention_mask.data<float>();
     }
+    TT_ENFORCE_EQ(seq, key_seq, "the fused core is for self attention without a key/value cache");
     const int32_t* cu = nullptr;
     if (seq_list != nullptr) cu = DeviceContext::GetInstance().GetSeqPlan(*seq_list).cu_seqlens;
-    TT_DEVICE_CALL(ttmi_fused_attention(q_.raw(), k_.raw(), v_.raw(), mask, ctx_.mutable_raw(), cu, batch, heads, seq, d,
+    TT_DEVICE_CALL(ttmi_fused_attention(q_.raw(), k.raw(), v.raw(), mask, ctx_.mutable_raw(), cu, batch, heads, seq, d,
                                         v_pitch, scaler, dt, Stream()));
   } else {
   Tensor* score = att_score != nullptr ? att_score : &score_scratch_;
-  score->ReshapeAs(query_tensor.dtype(), {batch, heads, seq, seq}, dev, dev_id, "batch_gemm3/Reshape");
+  // score is [B,h,F,T]: F = query positions, T = key positions (they differ for context attention
+  // and when a key/value cache has been prepended)
+  const int64_t F = seq, T = key_seq;
+  score->ReshapeAs(query_tensor.dtype(), {batch, heads, F, T}, dev, dev_id, "batch_gemm3/Reshape");
   // batch_gemm3: score[b,h] = scaler * q[b,h] k[b,h]^T   (multi_headed_attention.cpp:328-330)
-  TT_DEVICE_CALL(ttmi_gemm_strided_batched(q_.raw(), k_.raw(), score->mutable_raw(), seq, seq, d, d, d, seq, seq * d,
-                                           seq * d, seq * seq, batch * heads, 1, scaler, 0.f, dt, Stream()));
+  TT_DEVICE_CALL(ttmi_gemm_strided_batched(q_.raw(), k.raw(), score->mutable_raw(), F, T, d, d, d, T, F * d, T * d, F * T,
+                                           batch * heads, 1, scaler, 0.f, dt, Stream()));
   kernels::ApplyMaskAndSoftmax(score, attention_mask, 1.0f);
 
   if (seq_list == nullptr) {
-    // batch_gemm4 with the [B,h,S,d] -> [B,S,h,d] transpose folded into the store (:345-354)
-    TT_DEVICE_CALL(ttmi_gemm_batched_heads(score->raw(), v_.raw(), ctx_.mutable_raw(), seq, d, seq, seq, d, hidden, heads,
-                                           heads * seq * seq, seq * seq, heads * seq * d, seq * d, seq * hidden, d, batch, 0,
-                                           1.f, 0.f, dt, Stream()));
+    // batch_gemm4 with the [B,h,F,d] -> [B,F,h,d] transpose folded into the store (:345-354)
+    TT_DEVICE_CALL(ttmi_gemm_batched_heads(score->raw(), v.raw(), ctx_.mutable_raw(), F, d, T, T, d, hidden, heads,
+                                           heads * F * T, F * T, heads * T * d, T * d, F * hidden, d, batch, 0, 1.f, 0.f, dt,
+                                           Stream()));
   } else {
     // padded P V, then drop the pad rows while merging heads (…smart_batch.cpp:385-392)
     Tensor& padded = ln_query_;  // free at this point of the call
     padded.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "ApplyMaskAndSoftmax/Reshape");
-    TT_DEVICE_CALL(ttmi_gemm_strided_batched(score->raw(), v_.raw(), padded.mutable_raw(), seq, d, seq, seq, d, d, seq * seq,
+    TT_DEVICE_CALL(ttmi_gemm_strided_batched(score->raw(), v.raw(), padded.mutable_raw(), seq, d, seq, seq, d, d, seq * seq,
                                              seq * d, seq * d, batch * heads, 0, 1.f, 0.f, dt, Stream()));
     kernels::TransposeForScorePad(&ctx_, padded, *seq_list);
   }
@@ -110,59 +114,146 @@ void MultiHeadedAttention::SelfAttentionTail(const Tensor& query_tensor, const T
   }
 }
 
+// One projection followed by AddBiasTransposeForScore, as one GEMM: x[B,S,H] W + b -> [B,h,S,d]
+// (multi_headed_attention.cpp:73-88, :107-150).
+static void ProjectToHeads(const Tensor& x, const void* packed_w, const Tensor& bias, int64_t heads, Tensor* out,
+                           const char* name) {
+  const int64_t batch = x.shape(0), seq = x.shape(1), hidden = x.shape(2), d = hidden / heads;
+  out->ReshapeAs(x.dtype(), {batch, heads, seq, d}, x.device_type(), x.device_id(), name);
+  ttmi_epilogue_args args{};
+  args.bias = bias.raw();
+  args.q = out->mutable_raw();
+  args.seq = seq;
+  args.heads = heads;
+  args.head_dim = d;
+  TT_DEVICE_CALL(ttmi_gemm_fused(x.raw(), packed_w, nullptr, batch * seq, hidden, hidden, hidden, hidden, hidden,
+                                 TTMI_EPI_QKV_SPLIT, &args, kernels::DeviceDType(x), Stream()));
+}
+
+static bool CacheHas(const std::unordered_map<std::string, Tensor*>& cache, const char* key) {
+  auto it = cache.find(key);
+  return it != cache.end() && it->second != nullptr && !it->second->is_null();
+}
+
+// cache[key] = a copy of `src` (multi_headed_attention.cpp:216-229)
+static void StoreInCache(std::unordered_map<std::string, Tensor*>& cache, const char* key, const Tensor& src, const char* name) {
+  auto it = cache.find(key);
+  TT_ENFORCE(it != cache.end() && it->second != nullptr, "layer_cache has no entry %s", key);
+  std::vector<int64_t> shape;
+  for (size_t i = 0; i < src.n_dim(); ++i) shape.push_back(src.shape((int)i));
+  it->second->ReshapeAs(src.dtype(), shape, src.device_type(), src.device_id(), name);
+  core::CopyBytes(it->second->mutable_raw(), src.device_type(), src.raw(), src.device_type(),
+                  (size_t)src.numel() * src.element_size());
+}
+
 void MultiHeadedAttention::operator()(const Tensor& key_tensor, const Tensor& value_tensor, const Tensor& query_tensor,
                                       const Tensor& attention_mask, const std::string& attn_type, Tensor* output,
                                       Tensor* att_score, std::unordered_map<std::string, Tensor*> layer_cache,
                                       bool pre_layernorm, bool post_layernorm, bool post_add_input,
                                       bool is_trans_weight) const {
   std::lock_guard<std::mutex> g(mutex_);
-  TT_ENFORCE(attn_type == "self", "only attn_type \"self\" is built (\"context\" belongs to the decoder path)");
-  TT_ENFORCE(layer_cache.empty(), "layer_cache belongs to the decoder path and is not built");
+  const bool is_self = attn_type == "self";
+  TT_ENFORCE(is_self || attn_type == "context", "attn_type should be context or self.");
   TT_ENFORCE_EQ(query_tensor.n_dim(), (size_t)3, "The query_tensors should be a matrix with shape [batch_size, query_seq_len, hidden_size].");
   TT_ENFORCE(output != nullptr, "output must not be null");
   kernels::RequireGpu(query_tensor, "MultiHeadedAttention");
-  MultiHeadedAttention::EnforceShapeAndType();
-  (void)key_tensor;
-  (void)value_tensor;
+  TT_ENFORCE_EQ(dense_weight_.n_dim(), (size_t)2, "dense_weight must be a matrix");
 
   const int64_t batch = query_tensor.shape(0), seq = query_tensor.shape(1), hidden = query_tensor.shape(2);
   TT_ENFORCE_EQ(hidden, dense_weight_.shape(0), "hidden size of the input and of the weights differ");
-  TT_ENFORCE(core::SameDataType(query_tensor.dtype(), qkv_weight_.dtype()), "input and weights must share one element type");
+  TT_ENFORCE(core::SameDataType(query_tensor.dtype(), dense_weight_.dtype()), "input and weights must share one element type");
   const int64_t heads = num_attention_heads_, d = hidden / heads;
+  TT_ENFORCE(heads > 0 && hidden % heads == 0, "hidden must be a multiple of the head count");
   const int dt = kernels::DeviceDType(query_tensor);
   const DLDeviceType dev = query_tensor.device_type();
   const int dev_id = query_tensor.device_id();
+  for (const auto& kv : layer_cache) {
+    if (kv.second == nullptr || kv.second->is_null()) continue;
+    kernels::RequireGpu(*kv.second, "layer_cache");
+    TT_ENFORCE(core::SameDataType(kv.second->dtype(), query_tensor.dtype()), "layer_cache[%s] and the query differ in element type", kv.first.c_str());
+    TT_ENFORCE(kv.second->n_dim() == 4 && kv.second->shape(0) == batch && kv.second->shape(1) == heads && kv.second->shape(3) == d,
+               "layer_cache[%s] must be [batch, heads, len, head_dim]", kv.first.c_str());
+  }
 
-  const Tensor* qkv_in = &query_tensor;
-  if (pre_layernorm) {
-    TT_ENFORCE(!layernorm_gamma_.is_null(), "pre_layernorm needs LayerNorm parameters");
+  const Tensor* q_in = &query_tensor;
+  if (pre_layernorm) {  // :66-80, :190-199 -- eps is 1e-6 there
+    TT_ENFORCE(!layernorm_gamma_.is_null() && !layernorm_beta_.is_null(), "pre_layernorm needs LayerNorm parameters");
     ln_query_.ReshapeAs(query_tensor.dtype(), {batch, seq, hidden}, dev, dev_id, "self/layernorm/Reshape");
     core::CopyBytes(ln_query_.mutable_raw(), dev, query_tensor.raw(), dev, (size_t)query_tensor.numel() * query_tensor.element_size());
     kernels::LayerNorm<float>(layernorm_gamma_, layernorm_beta_, &ln_query_, 1e-6f);
-    qkv_in = &ln_query_;
+    q_in = &ln_query_;
   }
 
-  // with the fused core V is kept transposed, [B,h,d,pitch]: its tiles are then plain copies
-  const int64_t v_pitch = UseFusedCore(attention_mask, att_score, d, dt) ? RoundUp8(seq) : 0;
-  q_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/q/Reshape");
-  k_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/k/Reshape");
-  if (v_pitch > 0) v_.ReshapeAs(query_tensor.dtype(), {batch, heads, d, v_pitch}, dev, dev_id, "self/v/Reshape");
-  else v_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/v/Reshape");
-  // gemm012_fused + SplitAddBiasTransposeForScore in one launch (:199-203)
-  ttmi_epilogue_args args{};
-  args.bias = qkv_bias_.raw();
-  args.q = q_.mutable_raw();
-  args.k = k_.mutable_raw();
-  args.v = v_.mutable_raw();
-  args.seq = seq;
-  args.heads = heads;
-  args.head_dim = d;
-  args.v_seq_pitch = v_pitch;
-  TT_DEVICE_CALL(ttmi_gemm_fused(qkv_in->raw(), qkv_packed_.Get(qkv_weight_, is_trans_weight), nullptr, batch * seq, 3 * hidden,
-                                 hidden, hidden, hidden, 3 * hidden, TTMI_EPI_QKV_SPLIT, &args, dt, Stream()));
+  const Tensor* k_used = &k_;
+  const Tensor* v_used = &v_;
+  int64_t v_pitch = 0;
+  if (is_self) {
+    MultiHeadedAttention::EnforceShapeAndType();
+    // with the fused core V is kept transposed, [B,h,d,pitch]: its tiles are then plain copies.
+    // A key/value cache needs the row-major layout (it is appended along the sequence).
+    if (layer_cache.empty() && UseFusedCore(attention_mask, att_score, d, dt)) v_pitch = RoundUp8(seq);
+    q_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/q/Reshape");
+    k_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/k/Reshape");
+    if (v_pitch > 0) v_.ReshapeAs(query_tensor.dtype(), {batch, heads, d, v_pitch}, dev, dev_id, "self/v/Reshape");
+    else v_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/v/Reshape");
+    // gemm012_fused + SplitAddBiasTransposeForScore in one launch (:199-203)
+    ttmi_epilogue_args args{};
+    args.bias = qkv_bias_.raw();
+    args.q = q_.mutable_raw();
+    args.k = k_.mutable_raw();
+    args.v = v_.mutable_raw();
+    args.seq = seq;
+    args.heads = heads;
+    args.head_dim = d;
+    args.v_seq_pitch = v_pitch;
+    TT_DEVICE_CALL(ttmi_gemm_fused(q_in->raw(), qkv_packed_.Get(qkv_weight_, is_trans_weight), nullptr, batch * seq, 3 * hidden,
+                                   hidden, hidden, hidden, 3 * hidden, TTMI_EPI_QKV_SPLIT, &args, dt, Stream()));
+    // decoder self attention: earlier keys/values come first (:205-214), the grown tensors go back (:216-229)
+    auto prepend = [&](const char* key, Tensor* cur, Tensor* grown, const char* name) {
+      if (!CacheHas(layer_cache, key)) return;
+      const Tensor& past = *layer_cache.at(key);
+      const int64_t past_len = past.shape(2);
+      grown->ReshapeAs(query_tensor.dtype(), {batch, heads, past_len + seq, d}, dev, dev_id, name);
+      TT_DEVICE_CALL(ttmi_concat(past.raw(), cur->raw(), grown->mutable_raw(), batch * heads, past_len * d, seq * d, dt, Stream()));
+      std::swap(*cur, *grown);
+    };
+    prepend("self_keys", &k_, &k_grown_, "self/keys/Concat");
+    prepend("self_values", &v_, &v_grown_, "self/values/Concat");
+    if (!layer_cache.empty()) {
+      StoreInCache(layer_cache, "self_keys", k_, "self/self_key/Reshape");
+      StoreInCache(layer_cache, "self_values", v_, "self/self_value/Reshape");
+    }
+  } else {
+    TT_ENFORCE(!q_weight_.is_null() && !k_weight_.is_null() && !v_weight_.is_null() && !q_bias_.is_null() && !k_bias_.is_null() &&
+                   !v_bias_.is_null(), "context attention needs the separate q/k/v weights and biases");
+    ProjectToHeads(*q_in, q_packed_.Get(q_weight_, is_trans_weight), q_bias_, heads, &q_, "context/AddBiasTransposeForScore/q_out2/Reshape");
+    if (CacheHas(layer_cache, "memory_keys") && CacheHas(layer_cache, "memory_values")) {
+      // the encoder memory was projected at an earlier step (:90-105); used in place, no copy
+      k_used = layer_cache.at("memory_keys");
+      v_used = layer_cache.at("memory_values");
+    } else {
+      TT_ENFORCE_EQ(key_tensor.n_dim(), (size_t)3, "The key_tensor should be a matrix with shape [batch_size, key_seq_len, hidden_size].");
+      TT_ENFORCE_EQ(value_tensor.n_dim(), (size_t)3, "The value_tensor should be a matrix with shape [batch_size, key_seq_len, hidden_size].");
+      kernels::RequireGpu(key_tensor, "MultiHeadedAttention");
+      kernels::RequireGpu(value_tensor, "MultiHeadedAttention");
+      TT_ENFORCE(key_tensor.shape(0) == batch && value_tensor.shape(0) == batch && key_tensor.shape(1) == value_tensor.shape(1) &&
+                     key_tensor.shape(2) == hidden && value_tensor.shape(2) == hidden,
+                 "key and value must be [batch_size, key_seq_len, hidden_size]");
+      TT_ENFORCE(core::SameDataType(key_tensor.dtype(), query_tensor.dtype()) && core::SameDataType(value_tensor.dtype(), query_tensor.dtype()),
+                 "key, value and query must share one element type");
+      ProjectToHeads(key_tensor, k_packed_.Get(k_weight_, is_trans_weight), k_bias_, heads, &k_, "context/keys/AddBiasTransposeForScore/Reshape");
+      ProjectToHeads(value_tensor, v_packed_.Get(v_weight_, is_trans_weight), v_bias_, heads, &v_, "context/values/AddBiasTransposeForScore/Reshape");
+      if (!layer_cache.empty()) {  // :128-150
+        StoreInCache(layer_cache, "memory_keys", k_, "context/keys/AddBiasTransposeForScore/Reshape");
+        StoreInCache(layer_cache, "memory_values", v_, "context/values/AddBiasTransposeForScore/Reshape");
+      }
+    }
+  }
+  const int64_t key_seq = v_pitch > 0 ? seq : k_used->shape(2);
+  TT_ENFORCE_EQ(v_pitch > 0 ? seq : v_used->shape(2), key_seq, "keys and values differ in length");
 
-  SelfAttentionTail(query_tensor, attention_mask, output, att_score, batch, seq, nullptr, v_pitch, post_layernorm,
-                    post_add_input, is_trans_weight);
+  AttentionTail(query_tensor, attention_mask, output, att_score, batch, seq, key_seq, *k_used, *v_used, nullptr, v_pitch,
+                post_layernorm, post_add_input, is_trans_weight);
 }
 
 void BertAttention::operator()(const Tensor& input_tensor, const Tensor& attention_mask, Tensor* output, Tensor* attn,
@@ -231,8 +322,8 @@ void MultiHeadedAttentionSmartBatch::operator()(const Tensor& key_tensor, const 
   TT_DEVICE_CALL(ttmi_gemm_fused(query_tensor.raw(), qkv_packed_.Get(qkv_weight_, is_trans_weight), nullptr, plan.total,
                                  3 * hidden, hidden, hidden, hidden, 3 * hidden, TTMI_EPI_QKV_SPLIT_PAD, &args, dt, Stream()));
 
-  SelfAttentionTail(query_tensor, attention_mask, output, att_score, batch, max_seq, &query_seq_len_list, v_pitch,
-                    post_layernorm, post_add_input, is_trans_weight);
+  AttentionTail(query_tensor, attention_mask, output, att_score, batch, max_seq, max_seq, k_, v_, &query_seq_len_list, v_pitch,
+                post_layernorm, post_add_input, is_trans_weight);
 }
 
 }  // namespace layers

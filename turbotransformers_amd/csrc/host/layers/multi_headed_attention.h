@@ -3,8 +3,9 @@
 //   layers::MultiHeadedAttention            turbo_transformers/layers/multi_headed_attention.h:25-129
 //   layers::BertAttention                   turbo_transformers/layers/bert_attention.h:25-47
 //   layers::MultiHeadedAttentionSmartBatch  turbo_transformers/layers/multi_headed_attention_smart_batch.h:25-137
-// Only the self-attention path the BERT encoder uses is built ("context" attention and the
-// decoder's layer_cache belong to the OpenNMT decoder and raise an error).
+// MultiHeadedAttention also covers the decoder-side forms of the reference class: "context"
+// attention over an encoder memory (separate q/k/v projections, memory_keys/memory_values cache),
+// self attention with a growing self_keys/self_values cache, pre-LayerNorm and post_add_input.
 //
 // Device pipeline of one call (9 -> 6 launches by folding the memory-bound ops into GEMM
 // epilogues):
@@ -50,8 +51,9 @@ class MultiHeadedAttention {
 
   void EnforceShapeAndType() const;
 
-  // key/value/query [B,S,H]; attention_mask [B,1,1,S] (additive fp32) or empty;
-  // output [B,S,H]; att_score [B,h,S,S] (may be nullptr: then the probabilities stay internal).
+  // query [B,F,H]; key/value [B,T,H] (read by "context" attention only); attention_mask additive fp32,
+  // [B,1,1,T] / [B,1,T] (per key) or [B,F,T], or empty; output [B,F,H]; att_score [B,h,F,T] (may be
+  // nullptr: then the probabilities stay internal).  layer_cache entries are [B,h,len,d] or empty.
   void operator()(const core::Tensor& key_tensor, const core::Tensor& value_tensor, const core::Tensor& query_tensor,
                   const core::Tensor& attention_mask, const std::string& attn_type, core::Tensor* output,
                   core::Tensor* att_score, std::unordered_map<std::string, core::Tensor*> layer_cache,
@@ -60,10 +62,12 @@ class MultiHeadedAttention {
 
  protected:
   // Everything after q/k/v exist, shared by the dense and the smart-batch layers.
-  // `v_pitch` > 0: v_ holds V transposed, [B,h,d,v_pitch], and the fused attention kernel runs.
-  void SelfAttentionTail(const core::Tensor& query_tensor, const core::Tensor& attention_mask, core::Tensor* output,
-                         core::Tensor* att_score, int64_t batch, int64_t seq, const std::vector<int64_t>* seq_list,
-                         int64_t v_pitch, bool post_layernorm, bool post_add_input, bool is_trans_weight) const;
+  // `v_pitch` > 0: v holds V transposed, [B,h,d,v_pitch], and the fused attention kernel runs.
+  // `seq` query positions against `key_seq` key positions held in k / v ([B,h,key_seq,d]).
+  void AttentionTail(const core::Tensor& query_tensor, const core::Tensor& attention_mask, core::Tensor* output,
+                     core::Tensor* att_score, int64_t batch, int64_t seq, int64_t key_seq, const core::Tensor& k,
+                     const core::Tensor& v, const std::vector<int64_t>* seq_list, int64_t v_pitch, bool post_layernorm,
+                     bool post_add_input, bool is_trans_weight) const;
   // The whole attention core runs as one kernel when nobody asks for the probabilities
   // (fp16/bf16, head size 64, additive key mask broadcast over the query rows).
   static bool UseFusedCore(const core::Tensor& attention_mask, const core::Tensor* att_score, int64_t head_dim, int dtype);
@@ -73,9 +77,9 @@ class MultiHeadedAttention {
   core::Tensor layernorm_gamma_, layernorm_beta_;
   int64_t num_attention_heads_;
 
-  PackedWeight qkv_packed_, dense_packed_;
+  PackedWeight qkv_packed_, dense_packed_, q_packed_, k_packed_, v_packed_;
   // Per-call intermediates, reused across calls (Reshape keeps a buffer that is large enough).
-  mutable core::Tensor q_, k_, v_, ctx_, score_scratch_, ln_query_;
+  mutable core::Tensor q_, k_, v_, k_grown_, v_grown_, ctx_, score_scratch_, ln_query_;
   mutable std::mutex mutex_;  // the layer keeps per-call state, like the reference (…attention.cpp:32,272)
 };
 

@@ -244,6 +244,29 @@ def test_gemm_i8_accumulators_bit_exact(ttmi, oracle, M, N, K):
         assert np.array_equal(want, oracle.gemm_i8(A, B))
 
 
+@pytest.mark.parametrize("M,N,K,with_bias", [(2560, 768, 768, False), (2560, 3072, 768, True), (37, 100, 48, True), (300, 1000, 130, False)])
+def test_gemm_i8_dequant_equals_unfused(ttmi, oracle, M, N, K, with_bias):
+    """The dequantisation folded into the int8 GEMM gives the bits of gemm_i8 + dequant_bias, and those
+    are the oracle's scheme: float(acc) * s_x * s_w[n] (+ b[n])."""
+    rng = np.random.default_rng(M + N)
+    a = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    b = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    sx = np.array([0.0123, 0.0], np.float32)
+    sw = (rng.random(N, np.float32) + 0.5) * 1e-3
+    bias = rng.standard_normal(N).astype(np.float32) if with_bias else None
+    dA, dB, dsx, dsw = dev(a), dev(b), dev(sx), dev(sw)
+    dbias = dev(bias) if with_bias else None
+    acc = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    two_step, fused = torch.empty((M, N), device="cuda"), torch.empty((M, N), device="cuda")
+    ok(ttmi.ttmi_gemm_i8(ptr(dA), ptr(dB), ptr(acc), M, N, K, K, K, N, stream()))
+    ok(ttmi.ttmi_dequant_bias(ptr(acc), ptr(dsx), ptr(dsw), ptr(dbias) if with_bias else None, ptr(two_step), M, N, stream()))
+    ok(ttmi.ttmi_gemm_i8_dequant(ptr(dA), ptr(dB), ptr(fused), ptr(dsx), ptr(dsw), ptr(dbias) if with_bias else None, M, N, K, K,
+                                 K, N, stream()))
+    assert np.array_equal(host(fused), host(two_step))
+    want = oracle.dequant_bias(oracle.gemm_i8(a, b), sx[0], sw, bias if with_bias else np.zeros(N, np.float32))
+    assert max_abs(host(fused), want) <= 1e-5 * max(1.0, float(np.abs(want).max()))
+
+
 def test_int8_linear_pipeline(ttmi, oracle):
     """quantize -> int8 GEMM -> dequant+bias, against the oracle's statement of the same scheme."""
     rng = np.random.default_rng(3)

@@ -96,7 +96,7 @@ __device__ __forceinline__ int vt_pos(int within16) {
 }
 
 template <typename T, bool PACKED, bool VT>
-__global__ __launch_bounds__(256, 2) void fused_attention_kernel(const T* __restrict__ q, const T* __restrict__ k,
+__global__ __launch_bounds__(256, 4) void fused_attention_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                                  const T* __restrict__ v, const float* __restrict__ mask,
                                                                  T* __restrict__ out, const int32_t* __restrict__ cu,
                                                                  int heads, int seq, int v_pitch, float scale_log2e,

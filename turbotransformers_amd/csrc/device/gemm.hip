@@ -330,6 +330,38 @@ struct EpiInt32 {
   }
 };
 
+// int32 accumulators -> fp32: out = float(acc) * act_scale * w_scale[n] (+ bias[n]), the dequantisation
+// of the int8 Linear folded into the int8 GEMM.  The operation order is that of the stand-alone
+// dequant_bias kernel, so both give the same bits.
+struct EpiDequant {
+  using Acc = int;
+  float* c;
+  const float* act_scale;  // device scalar
+  const float* w_scale;    // [N]
+  const float* bias;       // [N] or null
+  int64_t ldc;
+  bool vec;
+  __device__ __forceinline__ const float* bias_ptr() const { return nullptr; }  // added after scaling, below
+  __device__ __forceinline__ void store8(int, int m, int n, int (&v)[8], int valid) const {
+    const float sx = act_scale[0];
+    float r[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      r[j] = 0.f;
+      if (j < valid) {
+        r[j] = (float)v[j] * sx * w_scale[n + j];
+        if (bias) r[j] += bias[n + j];
+      }
+    }
+    float* p = c + (int64_t)m * ldc + n;
+    if (vec && valid == 8) {
+      store_row8<float>(p, r);
+    } else {
+      for (int j = 0; j < valid; ++j) p[j] = r[j];
+    }
+  }
+};
+
 // -------------------------------------------------------------------------- kernel ------
 // LDS rows are 128 bytes and the LDS has 64 four-byte banks (256 bytes per bank cycle): rows r and
 // r+2 start on the same bank.  A 128-bit operand read is served 16 lanes (= 16 consecutive tile
@@ -1054,6 +1086,23 @@ int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_
   g.lda = lda; g.ldb = ldb;
   g.inner = 1;
   EpiInt32 epi{c, ldc, aligned16(c) && ldc % 4 == 0};
+  const bool aligned = aligned16(a) && aligned16(b) && lda % 16 == 0 && ldb % 16 == 0 && k % 16 == 0;
+  return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
+}
+
+int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev, const float* w_scale,
+                         const float* bias, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc,
+                         void* stream) {
+  TTMI_REQUIRE(a && b && c && act_scale_dev && w_scale, "null tensor");
+  TTMI_REQUIRE(m < (1ll << 31) && n < (1ll << 31) && k < (1ll << 31), "dimension too large");
+  TTMI_REQUIRE(lda >= k && ldb >= k && ldc >= n, "leading dimension too small");
+  GemmArgs g{};
+  g.a = (const char*)a;
+  g.b = (const char*)b;
+  g.m = (int)m; g.n = (int)n; g.k = (int)k;
+  g.lda = lda; g.ldb = ldb;
+  g.inner = 1;
+  EpiDequant epi{c, act_scale_dev, w_scale, bias, ldc, aligned16(c) && ldc % 4 == 0};
   const bool aligned = aligned16(a) && aligned16(b) && lda % 16 == 0 && ldb % 16 == 0 && k % 16 == 0;
   return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
 }

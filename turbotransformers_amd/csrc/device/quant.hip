@@ -12,6 +12,14 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ x
   float mx = 0.f;
   int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {  // 16-byte loads over the aligned body
+    const int64_t n4 = n / 4;
+    for (int64_t j = i; j < n4; j += stride) {
+      const float4 v = reinterpret_cast<const float4*>(x)[j];
+      mx = fmaxf(fmaxf(mx, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+    }
+    i += n4 * 4;
+  }
   for (; i < n; i += stride) mx = fmaxf(mx, fabsf(x[i]));
   mx = group_max<kWave>(mx);
   if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = mx;
@@ -98,7 +106,9 @@ int ttmi_quantize_rows_i8(const float* x, int8_t* q, float* scale_dev, int64_t m
   hipStream_t s = (hipStream_t)stream;
   int rc = ttmi_memset_zero(scale_dev, 2 * sizeof(float), stream);
   if (rc != 0) return rc;
-  hipLaunchKernelGGL(absmax_kernel, dim3(flat_grid(n)), dim3(256), 0, s, x, n, reinterpret_cast<uint32_t*>(scale_dev + 1));
+  // one atomic per workgroup on a single word: a few hundred workgroups keep that cheap
+  const unsigned absmax_grid = (unsigned)std::min<int64_t>(ceil_div(n, 256 * 16), 512);
+  hipLaunchKernelGGL(absmax_kernel, dim3(std::max(absmax_grid, 1u)), dim3(256), 0, s, x, n, reinterpret_cast<uint32_t*>(scale_dev + 1));
   hipLaunchKernelGGL(quantize_kernel, dim3(flat_grid(n)), dim3(256), 0, s, x, q, scale_dev, n);
   return launch_status("quantize_rows_i8");
 }

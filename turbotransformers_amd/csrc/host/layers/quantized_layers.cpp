@@ -40,15 +40,15 @@ void QuantizedLinear::operator()(const Tensor& input_tensor, Tensor* output_tens
   const DLDeviceType dev = input_tensor.device_type();
   const int id = input_tensor.device_id();
   int8_t* qx = q_input_.Reshape<int8_t>({m, k}, dev, id, "QuantizedLinear/q_input");
-  int32_t* acc = acc_.Reshape<int32_t>({m, n}, dev, id, "QuantizedLinear/acc");
   std::vector<int64_t> shape;
   for (size_t i = 0; i + 1 < input_tensor.n_dim(); ++i) shape.push_back(input_tensor.shape((int)i));
   shape.push_back(n);
   float* out = output_tensor->Reshape<float>(shape, dev, id, "QuantizedLinear/Reshape");
   float* scale = act_scale_.mutableData<float>();
   TT_DEVICE_CALL(ttmi_quantize_rows_i8(input_tensor.data<float>(), qx, scale, m, k, Stream()));
-  TT_DEVICE_CALL(ttmi_gemm_i8(qx, q_weight_.data<int8_t>(), acc, m, n, k, k, k, n, Stream()));
-  TT_DEVICE_CALL(ttmi_dequant_bias(acc, scale, w_scales_.data<float>(), nullptr, out, m, n, Stream()));
+  // int8 GEMM with the dequantisation folded into its store: the int32 accumulators stay on chip
+  TT_DEVICE_CALL(ttmi_gemm_i8_dequant(qx, q_weight_.data<int8_t>(), out, scale, w_scales_.data<float>(), nullptr, m, n, k, k, k,
+                                      n, Stream()));
 }
 
 void QuantizedBertAttention::operator()(const Tensor& input_tensor, const Tensor& attention_mask, Tensor* output,

@@ -48,6 +48,7 @@ __device__ __forceinline__ Chunk pack_chunk(const T (&tmp)[N]) {
 constexpr int kRowBytes = 128;   // bytes of K per LDS row and per K step
 constexpr int kChunks = 8;       // 16-byte chunks per LDS row
 constexpr int kNumXcd = 8;
+constexpr int kXcdRemapMinTiles = 32;  // below this a problem's tiles are not spread over the XCDs
 constexpr int kLdsPerCu = 160 * 1024;
 
 template <typename T>
@@ -464,8 +465,11 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
 
   // XCD-aware tile order: ids equal mod 8 run on one XCD; give each XCD a contiguous tile range.
   const int tiles = g.tiles_m * g.tiles_n;
+  // (with few tiles per problem -- typically many small batched problems -- the grid is one workgroup
+  // per tile: padding it to the XCD count would only launch idle workgroups)
+  const bool remap = tiles >= kXcdRemapMinTiles;
   const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
-  const int logical = (int)(blockIdx.x % kNumXcd) * per_xcd + (int)(blockIdx.x / kNumXcd);
+  const int logical = remap ? (int)(blockIdx.x % kNumXcd) * per_xcd + (int)(blockIdx.x / kNumXcd) : (int)blockIdx.x;
   if (logical >= tiles) return;
   int tile_m, tile_n;
   tile_coords(logical, g.tiles_m, g.tiles_n, tile_m, tile_n);
@@ -656,10 +660,12 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   // finished tile runs out of the other half of LDS, and the epilogue's global stores drain
   // under the next tile's K loop.
   const int tiles = g.tiles_m * g.tiles_n;
+  // With fewer than kXcdRemapMinTiles tiles per problem the grid is simply one workgroup per tile.
+  const bool remap = tiles >= kXcdRemapMinTiles;
   const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
-  const int xcd = (int)(blockIdx.x % kNumXcd), stride = (int)(gridDim.x / kNumXcd);
-  const int xcd_end = min((xcd + 1) * per_xcd, tiles);
-  int logical = xcd * per_xcd + (int)(blockIdx.x / kNumXcd);
+  const int xcd = (int)(blockIdx.x % kNumXcd), stride = remap ? (int)(gridDim.x / kNumXcd) : (int)gridDim.x;
+  const int xcd_end = remap ? min((xcd + 1) * per_xcd, tiles) : tiles;
+  int logical = remap ? xcd * per_xcd + (int)(blockIdx.x / kNumXcd) : (int)blockIdx.x;
   if (logical >= xcd_end) return;
   const int z = blockIdx.z;
   const T* A = reinterpret_cast<const T*>(g.a) + (int64_t)(z / g.inner) * g.a_outer + (int64_t)(z % g.inner) * g.a_inner;
@@ -816,7 +822,7 @@ static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   g.tiles_n = (g.n + BN - 1) / BN;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
   TTMI_REQUIRE(tiles < (1ll << 30) && batch < 65536, "GEMM grid too large");
-  const unsigned grid_x = (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd);
+  const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
   constexpr int DEPTH = (BM * BN <= 64 * 64 && ALIGNED) ? 2 : 1;
   auto kern = gemm_kernel<T, BM, BN, WM, WN, B_KN, ALIGNED, DEPTH, Epi>;
   if (LDS > 64 * 1024) {
@@ -853,7 +859,10 @@ static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   TTMI_REQUIRE(tiles < (1ll << 30) && batch < 65536, "GEMM grid too large");
   // as many workgroups as stay resident (LDS-limited), a multiple of the XCD count
   const int64_t resident = (int64_t)compute_units() * std::max(1, kLdsPerCu / LDS);
-  const unsigned grid_x = (unsigned)(std::min(ceil_div(tiles, kNumXcd), std::max<int64_t>(1, resident / kNumXcd)) * kNumXcd);
+  const unsigned grid_x =
+      tiles >= kXcdRemapMinTiles
+          ? (unsigned)(std::min(ceil_div(tiles, kNumXcd), std::max<int64_t>(1, resident / kNumXcd)) * kNumXcd)
+          : (unsigned)tiles;
   auto kern = gemm_fast_kernel<T, BM, BN, WM, WN, Epi>;
   if (LDS > 64 * 1024) {
     static bool attr_set = false;  // per instantiation

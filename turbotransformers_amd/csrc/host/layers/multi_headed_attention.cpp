@@ -48,7 +48,7 @@ static int64_t RoundUp8(int64_t n) { return (n + 7) / 8 * 8; }
 // score -> softmax -> P V -> merge heads -> output projection -> bias (+input) (+LayerNorm)
 void MultiHeadedAttention::AttentionTail(const Tensor& query_tensor, const Tensor& attention_mask, Tensor* output,
                                          Tensor* att_score, int64_t batch, int64_t seq, int64_t key_seq, const Tensor& k,
-                                         const Tensor& v, const std::vector<int64_t>* seq_list, int64_t v_pitch,
+                                         const Tensor& v, const std::vector<int64_t>* seq_list, bool fused_core, int64_t v_pitch,
                                          bool post_layernorm, bool post_add_input, bool is_trans_weight) const {
   const int dt = kernels::DeviceDType(query_tensor);
   const DLDeviceType dev = query_tensor.device_type();
@@ -61,7 +61,7 @@ void MultiHeadedAttention::AttentionTail(const Tensor& query_tensor, const Tenso
 
   // Nobody asked for the probabilities: run the whole core as one kernel; the [B,h,S,S] scores
   // never reach HBM.
-  if (v_pitch > 0) {
+  if (fused_core) {
     const float* mask = nullptr;
     if (!attention_mask.is_null()) {
       TT_ENFORCE_EQ(attention_mask.numel(), batch * seq, "attention mask has the wrong size");
@@ -252,7 +252,7 @@ void MultiHeadedAttention::operator()(const Tensor& key_tensor, const Tensor& va
   const int64_t key_seq = v_pitch > 0 ? seq : k_used->shape(2);
   TT_ENFORCE_EQ(v_pitch > 0 ? seq : v_used->shape(2), key_seq, "keys and values differ in length");
 
-  AttentionTail(query_tensor, attention_mask, output, att_score, batch, seq, key_seq, *k_used, *v_used, nullptr, v_pitch,
+  AttentionTail(query_tensor, attention_mask, output, att_score, batch, seq, key_seq, *k_used, *v_used, nullptr, v_pitch > 0, v_pitch,
                 post_layernorm, post_add_input, is_trans_weight);
 }
 
@@ -298,13 +298,14 @@ void MultiHeadedAttentionSmartBatch::operator()(const Tensor& key_tensor, const 
   // Padded q,k,v; the QKV GEMM scatters bias-added rows of the packed input into them.  The
   // unfused core multiplies whole padded tensors, so pad rows must be exactly 0 there
   // (transpose.cpp:504-522); the fused kernel never reads a pad row, so nothing is cleared.
-  const int64_t v_pitch = UseFusedCore(attention_mask, att_score, d, dt) ? RoundUp8(max_seq) : 0;
+  // V stays row-major here: sequences start at arbitrary packed rows, so a transposed store could
+  // rarely use 16-byte vectors, and that costs the QKV GEMM more than the scatter costs the attention kernel.
+  const bool fused_core = UseFusedCore(attention_mask, att_score, d, dt);
   Tensor* qkv[3] = {&q_, &k_, &v_};
   const char* names[3] = {"self/q/Reshape", "self/k/Reshape", "self/v/Reshape"};
   for (int i = 0; i < 3; ++i) {
-    if (i == 2 && v_pitch > 0) qkv[i]->ReshapeAs(query_tensor.dtype(), {batch, heads, d, v_pitch}, dev, dev_id, names[i]);
-    else qkv[i]->ReshapeAs(query_tensor.dtype(), {batch, heads, max_seq, d}, dev, dev_id, names[i]);
-    if (v_pitch > 0) continue;
+    qkv[i]->ReshapeAs(query_tensor.dtype(), {batch, heads, max_seq, d}, dev, dev_id, names[i]);
+    if (fused_core) continue;
     const size_t bytes = (size_t)qkv[i]->numel() * qkv[i]->element_size();
     TT_DEVICE_CALL(ttmi_memset_zero(qkv[i]->mutable_raw(), (bytes + 3) / 4 * 4  /* capacity is rounded to 512 B */, Stream()));
   }
@@ -318,11 +319,10 @@ void MultiHeadedAttentionSmartBatch::operator()(const Tensor& key_tensor, const 
   args.head_dim = d;
   args.token_rows = plan.token_rows;
   args.batch = batch;
-  args.v_seq_pitch = v_pitch;
   TT_DEVICE_CALL(ttmi_gemm_fused(query_tensor.raw(), qkv_packed_.Get(qkv_weight_, is_trans_weight), nullptr, plan.total,
                                  3 * hidden, hidden, hidden, hidden, 3 * hidden, TTMI_EPI_QKV_SPLIT_PAD, &args, dt, Stream()));
 
-  AttentionTail(query_tensor, attention_mask, output, att_score, batch, max_seq, max_seq, k_, v_, &query_seq_len_list, v_pitch,
+  AttentionTail(query_tensor, attention_mask, output, att_score, batch, max_seq, max_seq, k_, v_, &query_seq_len_list, fused_core, 0,
                 post_layernorm, post_add_input, is_trans_weight);
 }
 

@@ -62,11 +62,12 @@ class MultiHeadedAttention {
 
  protected:
   // Everything after q/k/v exist, shared by the dense and the smart-batch layers.
-  // `v_pitch` > 0: v holds V transposed, [B,h,d,v_pitch], and the fused attention kernel runs.
+  // `fused_core`: the one-kernel attention core runs; `v_pitch` > 0: v holds V transposed, [B,h,d,v_pitch].
   // `seq` query positions against `key_seq` key positions held in k / v ([B,h,key_seq,d]).
   void AttentionTail(const core::Tensor& query_tensor, const core::Tensor& attention_mask, core::Tensor* output,
                      core::Tensor* att_score, int64_t batch, int64_t seq, int64_t key_seq, const core::Tensor& k,
-                     const core::Tensor& v, const std::vector<int64_t>* seq_list, int64_t v_pitch, bool post_layernorm,
+                     const core::Tensor& v, const std::vector<int64_t>* seq_list, bool fused_core, int64_t v_pitch,
+                     bool post_layernorm,
                      bool post_add_input, bool is_trans_weight) const;
   // The whole attention core runs as one kernel when nobody asks for the probabilities
   // (fp16/bf16, head size 64, additive key mask broadcast over the query rows).

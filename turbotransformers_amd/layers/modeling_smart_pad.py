@@ -29,6 +29,23 @@ def smart_pad_mask(seq_len_list: Sequence[int]):
     return mask
 
 
+_POSITION_IDS_CACHE = {}
+
+
+def _packed_position_ids(lens, device):
+    """[1, sum(lens)] int64: 0..len-1 per request.  Built on the host in one piece and cached on the
+    list of lengths (one upload instead of one arange kernel per request)."""
+    key = (lens, str(device))
+    hit = _POSITION_IDS_CACHE.get(key)
+    if hit is None:
+        import numpy as np
+        if len(_POSITION_IDS_CACHE) >= 64:
+            _POSITION_IDS_CACHE.clear()
+        host = np.concatenate([np.arange(n, dtype=np.int64) for n in lens]).reshape(1, -1)
+        hit = _POSITION_IDS_CACHE[key] = torch.from_numpy(host).to(device)
+    return hit
+
+
 class MultiHeadedAttentionSmartBatch(cxx.MultiHeadedAttentionSmartBatch):
     def __call__(self, key_tensor: AnyTensor, value_tensor: AnyTensor, query_tensor: AnyTensor,
                  query_seq_len_list: Sequence[int], key_seq_len_list: Sequence[int], mask: Optional[AnyTensor] = None,
@@ -144,7 +161,7 @@ class BertModelNoPoolerSmartBatch:
         assert ids.numel() == sum(lens), "query_seq_len_list does not match the inputs"
         dev = ids.device
         if position_ids is None:  # each request counts its own positions from 0
-            position_ids = torch.cat([torch.arange(n, dtype=torch.int64, device=dev) for n in lens]).reshape(1, -1)
+            position_ids = _packed_position_ids(tuple(lens), dev)
         if token_type_ids is None:
             token_type_ids = torch.zeros_like(ids)
         hidden = self.embeddings(ids, position_ids=position_ids, token_type_ids=token_type_ids,

@@ -52,6 +52,43 @@ def test_matmul(ttmi, oracle, dt, b_trans, M, N, K):
 
 
 @pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("M,N,K", [(128, 768, 3072), (128, 768, 768), (1, 768, 3072), (100, 2304, 768), (200, 3072, 1024),
+                                   (64, 520, 4096)])
+def test_matmul_small_m_long_k(ttmi, oracle, dt, M, N, K):
+    """Few output tiles, long K: the split-K path (K slices summed in a fixed order by a second kernel).
+    Same bound as any other MatMul, and two runs give the same bits."""
+    rng = np.random.default_rng(M + N + K)
+    A, B = _ab(rng, M, N, K, 1)
+    dA, dB = dev(A, dt), dev(B, dt)
+    C1 = torch.empty((M, N), dtype=dA.dtype, device="cuda")
+    C2 = torch.empty_like(C1)
+    for C in (C1, C2):
+        ok(ttmi.ttmi_gemm(ptr(dA), ptr(dB), ptr(C), M, N, K, K, K, N, 1, 1.0, 0.0, TTMI_DTYPES[dt], stream()))
+    want = oracle.matmul(rounded(A, dt), rounded(B, dt), True)
+    assert max_abs(host(C1), want) <= GEMM_TOL[dt] * max(1.0, float(np.abs(want).max()))
+    assert torch.equal(C1, C2)
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+def test_fused_epilogues_small_m_long_k(ttmi, oracle, dt):
+    """bias + GELU and bias + residual through the split-K reduction kernel."""
+    import ctypes
+    rng = np.random.default_rng(5)
+    M, N, K = 96, 768, 3072
+    A, W = _ab(rng, M, N, K, 1)
+    bias, res = rng.standard_normal(N).astype(np.float32), rng.standard_normal((M, N)).astype(np.float32)
+    dA, dW, db, dres = dev(A, dt), dev(W, dt), dev(bias, dt), dev(res, dt)
+    base = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    C = torch.empty((M, N), dtype=dA.dtype, device="cuda")
+    ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, capi.EPI_BIAS_ACT,
+                            ctypes.byref(_epi(bias=db, act=capi.ACT_GELU)), TTMI_DTYPES[dt], stream()))
+    assert max_abs(host(C), oracle.add_bias_act(base, rounded(bias, dt), 0)) <= GEMM_TOL[dt] * 3
+    ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, capi.EPI_BIAS_RESIDUAL,
+                            ctypes.byref(_epi(bias=db, residual=dres)), TTMI_DTYPES[dt], stream()))
+    assert max_abs(host(C), base + rounded(bias, dt) + rounded(res, dt)) <= GEMM_TOL[dt] * 3
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
 def test_matmul_alpha_beta_and_ld(ttmi, oracle, dt):
     rng = np.random.default_rng(5)
     M, N, K, lda, ldb, ldc = 70, 90, 64, 80, 72, 96

@@ -21,6 +21,9 @@
 //
 // Block ids are remapped so that the workgroups resident on one XCD (ids equal mod 8)
 // cover neighbouring tiles and share A rows / the weight matrix in that XCD's L2.
+#include <map>
+#include <mutex>
+
 #include "common.h"
 
 namespace ttmi {
@@ -126,6 +129,7 @@ struct GemmArgs {
   int inner;
   int64_t a_outer, a_inner, b_outer, b_inner;
   int tiles_m, tiles_n;
+  int k_chunk;  // split-K: blockIdx.y owns K range [y*k_chunk, (y+1)*k_chunk) and z passed to the epilogue is y; 0 = whole K
 };
 
 // ------------------------------------------------------------------------ epilogues -----
@@ -478,6 +482,14 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
 
   const T* A = reinterpret_cast<const T*>(g.a) + (int64_t)(z / g.inner) * g.a_outer + (int64_t)(z % g.inner) * g.a_inner;
   const T* B = reinterpret_cast<const T*>(g.b) + (int64_t)(z / g.inner) * g.b_outer + (int64_t)(z % g.inner) * g.b_inner;
+  int kdim = g.k, z_epi = z;
+  if (g.k_chunk > 0) {  // split-K (NK layout only): this workgroup sums a slice of K into its own partial tile
+    const int k_lo = (int)blockIdx.y * g.k_chunk;
+    kdim = min(g.k_chunk, g.k - k_lo);
+    A += k_lo;
+    B += k_lo;
+    z_epi = (int)blockIdx.y;
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid % kWave, wave = tid / kWave;
@@ -516,16 +528,16 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
 #pragma unroll
     for (int i = 0; i < A_ITERS; ++i) {
       const int c = i * NT + tid;
-      ra[i] = load_chunk(A, g.lda, m0 + (c >> 3), g.m, k0 + (c & 7) * KPC, g.k);
+      ra[i] = load_chunk(A, g.lda, m0 + (c >> 3), g.m, k0 + (c & 7) * KPC, kdim);
     }
 #pragma unroll
     for (int i = 0; i < B_ITERS; ++i) {
       const int c = i * NT + tid;
       if (!B_KN) {
-        rb[i] = load_chunk(B, g.ldb, n0 + (c >> 3), g.n, k0 + (c & 7) * KPC, g.k);
+        rb[i] = load_chunk(B, g.ldb, n0 + (c >> 3), g.n, k0 + (c & 7) * KPC, kdim);
       } else {
         // B[K,N]: row = k index, columns = n
-        rb[i] = load_chunk(B, g.ldb, k0 + c / KN_CPR, g.k, n0 + (c % KN_CPR) * KPC, g.n);
+        rb[i] = load_chunk(B, g.ldb, k0 + c / KN_CPR, kdim, n0 + (c % KN_CPR) * KPC, g.n);
       }
     }
   };
@@ -583,7 +595,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
     }
   };
 
-  const int ksteps = (g.k + BK - 1) / BK;
+  const int ksteps = (kdim + BK - 1) / BK;
   load_global(0, ra[0], rb[0]);
   store_lds(0, ra[0], rb[0]);
   __syncthreads();
@@ -615,7 +627,58 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
 
   float bj[TN];
   load_bias_columns<TN>(epi, n0 + wn0 + lrow, g.n, bj);
-  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, bj, smem, epi, g, z, m0 + wm0, n0 + wn0, lane, wave);
+  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, bj, smem, epi, g, z_epi, m0 + wm0, n0 + wn0, lane, wave);
+}
+
+// ---------------------------------------------------------------------------- split-K -----
+// Few output tiles and a long K (one short sequence through the FFN: 24 tiles, 48..96 K steps)
+// leave most of the chip idle behind a long serial chain.  Then K is cut into `splits` slices,
+// every slice is an ordinary workgroup that stores its fp32 partial tile to a workspace
+// [splits][M][N], and a second small kernel sums the slices in a fixed order (so results are
+// reproducible) and applies the real epilogue.
+struct EpiPartial {
+  using Acc = float;
+  float* ws;
+  int64_t mn;   // M*N
+  int64_t ldn;  // N
+  bool vec;
+  __device__ __forceinline__ const float* bias_ptr() const { return nullptr; }
+  __device__ __forceinline__ void store8(int split, int m, int n, float (&v)[8], int valid) const {
+    float* p = ws + split * mn + (int64_t)m * ldn + n;
+    if (vec && valid == 8) {
+      store_row8<float>(p, v);
+    } else {
+      for (int j = 0; j < valid; ++j) p[j] = v[j];
+    }
+  }
+};
+
+template <typename Epi>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int m, int n, bool vec,
+                                                            const Epi epi) {
+  const int groups = (n + 7) / 8;
+  const int64_t idx = blockIdx.x * (int64_t)256 + threadIdx.x;
+  const int row = (int)(idx / groups), ncol = (int)(idx % groups) * 8;
+  if (row >= m) return;
+  const int valid = min(8, n - ncol);
+  float v[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = 0.f;
+  for (int sidx = 0; sidx < splits; ++sidx) {
+    const float* p = ws + ((int64_t)sidx * m + row) * n + ncol;
+    if (vec && valid == 8) {
+      float x[8];
+      load_row8<float>(p, x);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] += x[j];
+    } else {
+      for (int j = 0; j < valid; ++j) v[j] += p[j];
+    }
+  }
+  const auto* bias = epi.bias_ptr();
+  if (bias != nullptr)
+    for (int j = 0; j < valid; ++j) v[j] += to_float(bias[ncol + j]);
+  epi.store8(0, row, ncol, v, valid);
 }
 
 // ------------------------------------------------------------------ fast-path kernel -----
@@ -875,6 +938,61 @@ static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   return launch_status("gemm_fast_kernel");
 }
 
+// Workspace of the split-K path: one buffer per stream, grown on demand, kept for the life of
+// the process (work on one stream is ordered, so consecutive GEMMs can share it).
+static float* splitk_workspace(size_t bytes, hipStream_t s) {
+  struct Slot {
+    float* ptr = nullptr;
+    size_t bytes = 0;
+  };
+  static std::mutex mu;
+  static std::map<hipStream_t, Slot> slots;
+  std::lock_guard<std::mutex> lock(mu);
+  Slot& slot = slots[s];
+  if (slot.bytes < bytes) {
+    if (slot.ptr != nullptr) {
+      if (hipStreamSynchronize(s) != hipSuccess) return nullptr;
+      (void)hipFree(slot.ptr);
+      slot = Slot{};
+    }
+    const size_t want = std::max(bytes, (size_t)8 << 20);
+    void* p = nullptr;
+    if (hipMalloc(&p, want) != hipSuccess) return nullptr;
+    slot.ptr = static_cast<float*>(p);
+    slot.bytes = want;
+  }
+  return slot.ptr;
+}
+
+// Number of K slices for a small problem (1 = do not split): enough workgroups to cover the chip,
+// at least four K steps per slice.
+static int pick_splits(int64_t m, int64_t n, int64_t ksteps, int64_t batch) {
+  const int64_t tiles = ceil_div(m, 64) * ceil_div(n, 64);
+  if (batch != 1 || tiles > 128 || ksteps < 8) return 1;
+  return (int)std::max<int64_t>(1, std::min<int64_t>({(int64_t)compute_units() / tiles, ksteps / 4, 16}));
+}
+
+template <typename T, typename Epi>
+static int launch_splitk(GemmArgs g, const Epi& epi, int splits, int64_t ksteps, int bk, hipStream_t s) {
+  const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
+  float* ws = splitk_workspace(bytes, s);
+  TTMI_REQUIRE(ws != nullptr, "cannot allocate the split-K workspace");
+  g.k_chunk = (int)ceil_div(ksteps, splits) * bk;
+  const int used = (int)ceil_div(g.k, g.k_chunk);  // slices that actually hold part of K
+  g.tiles_m = (g.m + 63) / 64;
+  g.tiles_n = (g.n + 63) / 64;
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  const bool vec = g.n % 4 == 0;
+  EpiPartial part{ws, (int64_t)g.m * g.n, g.n, vec};
+  constexpr int LDS = 2 * (64 + 64) * kRowBytes;
+  const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
+  hipLaunchKernelGGL((gemm_kernel<T, 64, 64, 2, 2, false, true, 2, EpiPartial>), dim3(grid_x, (unsigned)used, 1), dim3(256), LDS, s,
+                     g, part);
+  const int64_t items = (int64_t)g.m * ((g.n + 7) / 8);
+  hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3((unsigned)ceil_div(items, 256)), dim3(256), 0, s, ws, used, g.m, g.n, vec, epi);
+  return launch_status("gemm_splitk");
+}
+
 // Tile configurations of the fast path and a cost model to pick one.  With t = tile area /
 // efficiency as the time of one tile on an otherwise idle CU, and `per_cu` workgroups of that
 // size resident per CU (they then share its MFMA pipes):
@@ -924,7 +1042,15 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
         case 3: return launch_fast<T, 128, 128, 2, 2, Epi>(g, epi, batch, s);
         // small problems are latency-bound: the register-staged kernel hides the global latency
         // of a one-step prefetch better than the DMA path does with a tiny tile
-        default: return launch_config<T, 64, 64, 2, 2, false, true, Epi>(g, epi, batch, s);
+        default: {
+          if constexpr (std::is_same<typename Epi::Acc, float>::value) {
+            bool column_pass = false;
+            if constexpr (HasColumnPass<Epi>::value) column_pass = epi.v_pitch > 0;
+            const int splits = column_pass ? 1 : pick_splits(g.m, g.n, g.k / BK, batch);
+            if (splits > 1) return launch_splitk<T, Epi>(g, epi, splits, g.k / BK, BK, s);
+          }
+          return launch_config<T, 64, 64, 2, 2, false, true, Epi>(g, epi, batch, s);
+        }
       }
     }
     if (aligned) {

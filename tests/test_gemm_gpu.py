@@ -53,7 +53,7 @@ def test_matmul(ttmi, oracle, dt, b_trans, M, N, K):
 
 @pytest.mark.parametrize("dt", ALL_DTYPES)
 @pytest.mark.parametrize("M,N,K", [(128, 768, 3072), (128, 768, 768), (1, 768, 3072), (100, 2304, 768), (200, 3072, 1024),
-                                   (64, 520, 4096)])
+                                   (64, 520, 4096), (2560, 768, 3072), (2048, 768, 3072), (1000, 1024, 4096)])
 def test_matmul_small_m_long_k(ttmi, oracle, dt, M, N, K):
     """Few output tiles, long K: the split-K path (K slices summed in a fixed order by a second kernel).
     Same bound as any other MatMul, and two runs give the same bits."""

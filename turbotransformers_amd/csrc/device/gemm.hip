@@ -742,7 +742,14 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   // byte offsets of this lane's operand rows inside a stage (swizzle folded in per k-substep)
   const int a_row0 = (wm0 + lrow) * kRowBytes, b_row0 = A_BYTES + (wn0 + lrow) * kRowBytes;
   const int swz = ((lrow >> 1) & 7);  // rows wm0 + 32 i + lrow share (row>>1)&7 with lrow
-  const int ksteps = g.k / BK;
+  int ksteps = g.k / BK, z_epi = z;
+  if (g.k_chunk > 0) {  // split-K: this workgroup multiplies one K slice into its own partial tile
+    const int k_lo = (int)blockIdx.y * g.k_chunk;
+    ksteps = min(g.k_chunk, g.k - k_lo) / BK;
+    A += k_lo;
+    B += k_lo;
+    z_epi = (int)blockIdx.y;
+  }
 
   // per-lane source pointers of the DMA loads (advanced by one K step per issue)
   const T* pa[A_LOADS];
@@ -869,8 +876,8 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
       point_at(next);
       issue(0);
     }
-    store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN>() - STAGE>(acc, bj, smem + STAGE, epi, g, z, m0 + wm0, n0 + wn0,
-                                                                         lane, wave);
+    store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN>() - STAGE>(acc, bj, smem + STAGE, epi, g, z_epi, m0 + wm0,
+                                                                         n0 + wn0, lane, wave);
     if (next >= xcd_end) break;
     logical = next;
   }
@@ -993,6 +1000,35 @@ static int launch_splitk(GemmArgs g, const Epi& epi, int splits, int64_t ksteps,
   return launch_status("gemm_splitk");
 }
 
+// Split-K on the DMA kernel with 128x128 tiles, for mid-size problems whose tiles do not fill the chip
+// (M = 2560, N = 768, K = 3072: 120 tiles, 48 K steps each).
+template <typename T, typename Epi>
+static int launch_fast_splitk(GemmArgs g, const Epi& epi, int splits, int64_t ksteps, int bk, hipStream_t s) {
+  const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
+  float* ws = splitk_workspace(bytes, s);
+  TTMI_REQUIRE(ws != nullptr, "cannot allocate the split-K workspace");
+  g.k_chunk = (int)ceil_div(ksteps, splits) * bk;
+  const int used = (int)ceil_div(g.k, g.k_chunk);
+  g.tiles_m = (g.m + 127) / 128;
+  g.tiles_n = (g.n + 127) / 128;
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  const bool vec = g.n % 4 == 0;
+  EpiPartial part{ws, (int64_t)g.m * g.n, g.n, vec};
+  constexpr int LDS = fast_lds_bytes<128, 128, 2, 2>();
+  auto kern = gemm_fast_kernel<T, 128, 128, 2, 2, EpiPartial>;
+  static bool attr_set = false;  // per instantiation
+  if (!attr_set) {
+    TTMI_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+    attr_set = true;
+  }
+  // one workgroup per (tile, slice): the persistent loop runs once
+  const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
+  hipLaunchKernelGGL(kern, dim3(grid_x, (unsigned)used, 1), dim3(256), LDS, s, g, part);
+  const int64_t items = (int64_t)g.m * ((g.n + 7) / 8);
+  hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3((unsigned)ceil_div(items, 256)), dim3(256), 0, s, ws, used, g.m, g.n, vec, epi);
+  return launch_status("gemm_fast_splitk");
+}
+
 // Tile configurations of the fast path and a cost model to pick one.  With t = tile area /
 // efficiency as the time of one tile on an otherwise idle CU, and `per_cu` workgroups of that
 // size resident per CU (they then share its MFMA pipes):
@@ -1039,7 +1075,18 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
         case 0: return launch_fast<T, 256, 256, 2, 4, Epi>(g, epi, batch, s);
         case 1: return launch_fast<T, 256, 192, 4, 2, Epi>(g, epi, batch, s);
         case 2: return launch_fast<T, 256, 128, 4, 2, Epi>(g, epi, batch, s);
-        case 3: return launch_fast<T, 128, 128, 2, 2, Epi>(g, epi, batch, s);
+        case 3: {
+          if constexpr (std::is_same<typename Epi::Acc, float>::value) {
+            bool column_pass = false;
+            if constexpr (HasColumnPass<Epi>::value) column_pass = epi.v_pitch > 0;
+            const int64_t ksteps = g.k / BK, t128 = tiles(128, 128);
+            if (!column_pass && batch == 1 && t128 <= compute_units() / 2 && ksteps >= 16) {
+              const int splits = (int)std::min<int64_t>({2 * (int64_t)compute_units() / t128, ksteps / 8, 8});
+              if (splits > 1) return launch_fast_splitk<T, Epi>(g, epi, splits, ksteps, BK, s);
+            }
+          }
+          return launch_fast<T, 128, 128, 2, 2, Epi>(g, epi, batch, s);
+        }
         // small problems are latency-bound: the register-staged kernel hides the global latency
         // of a one-step prefetch better than the DMA path does with a tiny tile
         default: {

@@ -27,6 +27,9 @@ DEVICE_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-I", INCLUDE,
 ]
+# Per-file additions.  attention.hip: maxima over MFMA results would otherwise be preceded by one
+# canonicalising v_max per operand (signalling-NaN quieting), a tenth of the softmax's VALU work.
+DEVICE_FILE_FLAGS = {"attention.hip": ["-fno-honor-nans"]}
 
 
 def _run(cmd):
@@ -69,7 +72,7 @@ def build_device(jobs=8, verbose=True, force=True):
         obj = os.path.join(OBJ_DIR, name[:-4] + ".o")
         if not force and not _stale(obj, [os.path.join(src_dir, name)] + headers):
             return obj
-        out = _run([HIPCC] + DEVICE_FLAGS + ["-c", os.path.join(src_dir, name), "-o", obj])
+        out = _run([HIPCC] + DEVICE_FLAGS + DEVICE_FILE_FLAGS.get(name, []) + ["-c", os.path.join(src_dir, name), "-o", obj])
         if verbose and out.strip():
             print(out)
         return obj

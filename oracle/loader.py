@@ -303,6 +303,25 @@ class Oracle:
             out = out + f32(w["dense_b"])
         return f32(out), attn
 
+    def positionwise_ffn(self, x, w1, b1, w2, b2, ln_g, ln_b):
+        """layers::PositionwiseFeedForward (layers/positionwise_ffn.cpp:33-77): LayerNorm (eps 1e-12), MatMul,
+        AddBiasAct<Relu>, MatMul, AddInputBias.  Weights [in, out]."""
+        x = np.ascontiguousarray(x, np.float32)
+        B, S, H = x.shape
+        normed = self.layer_norm(x, ln_g, ln_b, 1e-12)
+        hidden = self.add_bias_act(self.matmul(normed.reshape(B * S, H), np.ascontiguousarray(w1, np.float32)), b1, 2)
+        out = self.matmul(hidden, np.ascontiguousarray(w2, np.float32)).reshape(B, S, H)
+        return np.ascontiguousarray(out + x + np.asarray(b2, np.float32), np.float32)
+
+    def distill_ffn(self, x, w1, b1, w2, b2, ln_g, ln_b):
+        """layers::DistrillFFN (layers/positionwise_ffn.cpp:79-127): MatMul, AddBiasAct<Gelu>, MatMul,
+        AddInputBias, LayerNorm (eps 1e-12) -- the last two are exactly AddBiasLayerNorm."""
+        x = np.ascontiguousarray(x, np.float32)
+        B, S, H = x.shape
+        hidden = self.add_bias_act(self.matmul(x.reshape(B * S, H), np.ascontiguousarray(w1, np.float32)), b1, 0)
+        out = self.matmul(hidden, np.ascontiguousarray(w2, np.float32)).reshape(B, S, H)
+        return self.add_bias_layer_norm(out, x, b2, ln_g, ln_b, 1e-12)
+
     def bert_layer(self, x, mask, w, heads):
         B, S, H = x.shape
         F = w["inter_w"].shape[1]

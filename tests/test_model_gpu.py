@@ -604,3 +604,37 @@ def test_multi_headed_attention_rejects_bad_arguments(tt):
     bad = {"self_keys": torch.zeros(2, 4, 3, 32).cuda(), "self_values": torch.zeros(2, 4, 3, 64).cuda()}
     with pytest.raises(RuntimeError, match="layer_cache"):
         layer(x, x, x, layer_cache=bad, attn_type="self")
+
+
+class _OnmtLikeFfn(torch.nn.Module):
+    def __init__(self, hidden, d_ff):
+        super().__init__()
+        self.w_1, self.w_2 = torch.nn.Linear(hidden, d_ff), torch.nn.Linear(d_ff, hidden)
+        self.layer_norm = torch.nn.LayerNorm(hidden, eps=1e-12)
+        self.lin1, self.lin2 = self.w_1, self.w_2  # DistilBERT's names for the same two layers
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("is_trans_weight", [False, True])
+def test_feed_forward_blocks(tt, oracle, dtype, is_trans_weight):
+    """layers/positionwise_ffn.cpp:33-127: both blocks against the oracle's compositions."""
+    torch.manual_seed(11)
+    H, F, B, S = 256, 1024, 3, 17
+    mod = _OnmtLikeFfn(H, F).cuda()
+    with torch.no_grad():
+        mod.layer_norm.weight.normal_(1, 0.1)
+        mod.layer_norm.bias.normal_(0, 0.1)
+    mod = mod.to(dtype)
+    x = torch.randn(B, S, H, generator=torch.Generator().manual_seed(12)).cuda().to(dtype)
+    f = lambda t: host(t.detach().float())
+    args = (f(x), f(mod.w_1.weight).T.copy(), f(mod.w_1.bias), f(mod.w_2.weight).T.copy(), f(mod.w_2.bias),
+            f(mod.layer_norm.weight), f(mod.layer_norm.bias))
+    tol = 2e-4 if dtype == torch.float32 else 2e-2
+    pw = tt.PositionwiseFeedForward.from_onmt(mod, is_trans_weight=is_trans_weight)
+    got = pw(x, is_trans_weight=is_trans_weight)
+    assert got.dtype == dtype and max_abs(f(got), oracle.positionwise_ffn(*args)) < tol
+    df = tt.DistrillFFN.from_torch(mod, mod.layer_norm, is_trans_weight=is_trans_weight)
+    got = df(x, is_trans_weight=is_trans_weight)
+    assert got.dtype == dtype and max_abs(f(got), oracle.distill_ffn(*args)) < tol
+    with pytest.raises(RuntimeError, match="model_dim"):
+        pw(torch.zeros(1, 2, H + 8, device="cuda", dtype=dtype), is_trans_weight=is_trans_weight)

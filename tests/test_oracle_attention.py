@@ -108,3 +108,21 @@ def test_concat_and_single_projection_split(oracle):
     x, bias = rng.standard_normal((2, 7, 3, 4), np.float32), rng.standard_normal(12).astype(np.float32)
     got = oracle.add_bias_transpose_for_score(x, bias, 2, 7, 3, 4)
     assert np.array_equal(got, (x + bias.reshape(3, 4)).transpose(0, 2, 1, 3))
+
+
+def test_feed_forward_blocks_vs_torch(oracle):
+    """PositionwiseFeedForward / DistrillFFN compositions against the same mathematics in torch."""
+    torch.manual_seed(9)
+    H, F = 48, 160
+    lin1, lin2, ln = torch.nn.Linear(H, F), torch.nn.Linear(F, H), torch.nn.LayerNorm(H, eps=1e-12)
+    with torch.no_grad():
+        ln.weight.normal_(1, 0.1)
+        ln.bias.normal_(0, 0.1)
+    x = torch.randn(2, 5, H)
+    n = lambda t: t.detach().numpy().copy()
+    args = (n(x), n(lin1.weight).T.copy(), n(lin1.bias), n(lin2.weight).T.copy(), n(lin2.bias), n(ln.weight), n(ln.bias))
+    with torch.no_grad():
+        want_pw = x + lin2(torch.relu(lin1(ln(x))))
+        want_df = ln(x + lin2(torch.nn.functional.gelu(lin1(x), approximate="tanh")))
+    assert np.abs(oracle.positionwise_ffn(*args) - want_pw.numpy()).max() < 2e-5
+    assert np.abs(oracle.distill_ffn(*args) - want_df.numpy()).max() < 2e-5

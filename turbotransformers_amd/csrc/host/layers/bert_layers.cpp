@@ -154,6 +154,54 @@ SequencePool::SequencePool(const std::string& pool_type) {
 
 void SequencePool::operator()(const Tensor& input, Tensor* output) const { kernels::SeqPool(input, pool_type_, output); }
 
+static void CheckFfn(const Tensor& input, const Tensor& w1, const Tensor& b1, const Tensor& w2, const Tensor& b2, bool trans,
+                     const char* who) {
+  kernels::RequireGpu(input, who);
+  TT_ENFORCE_EQ(input.n_dim(), (size_t)3, "input should be [batch_size, input_len, model_dim]");
+  TT_ENFORCE(w1.n_dim() == 2 && w2.n_dim() == 2, "dense weights must be matrices");
+  TT_ENFORCE_EQ(PackedWeight::InDim(w1, trans), input.shape(2), "dense weight and input tensor should have the same model_dim.");
+  TT_ENFORCE_EQ(PackedWeight::InDim(w2, trans), PackedWeight::OutDim(w1, trans), "the two dense weights do not chain");
+  TT_ENFORCE_EQ(PackedWeight::OutDim(w2, trans), input.shape(2), "the second dense weight must map back to model_dim");
+  TT_ENFORCE_EQ(b1.numel(), PackedWeight::OutDim(w1, trans), "dense_bias_1 size mismatch");
+  TT_ENFORCE_EQ(b2.numel(), input.shape(2), "dense_bias_2 size mismatch");
+  TT_ENFORCE(core::SameDataType(input.dtype(), w1.dtype()), "input and weights must share one element type");
+}
+
+void PositionwiseFeedForward::operator()(const Tensor& input_tensor, Tensor* output, bool is_trans_weight) const {
+  CheckFfn(input_tensor, dense_weight_1_, dense_bias_1_, dense_weight_2_, dense_bias_2_, is_trans_weight, "PositionwiseFeedForward");
+  const int64_t model_dim = input_tensor.shape(2), d_ff = PackedWeight::OutDim(dense_weight_1_, is_trans_weight);
+  const int64_t m = input_tensor.numel() / model_dim;
+  const DLDeviceType dev = input_tensor.device_type();
+  const int id = input_tensor.device_id();
+  normed_.ReshapeAs(input_tensor.dtype(), {input_tensor.shape(0), input_tensor.shape(1), model_dim}, dev, id, "FFN/LayerNorm/Reshape");
+  core::CopyBytes(normed_.mutable_raw(), dev, input_tensor.raw(), dev, (size_t)input_tensor.numel() * input_tensor.element_size());
+  kernels::LayerNorm<float>(layer_norm_weight_, layer_norm_bias_, &normed_, 1e-12f);
+  hidden_.ReshapeAs(input_tensor.dtype(), {m, d_ff}, dev, id, "FFN/gemm0/Reshape");
+  GemmBiasAct(normed_, packed1_.Get(dense_weight_1_, is_trans_weight), d_ff, dense_bias_1_, TTMI_ACT_RELU, &hidden_);
+  output->ReshapeAs(input_tensor.dtype(), {input_tensor.shape(0), input_tensor.shape(1), model_dim}, dev, id, "FFN/Reshape");
+  // gemm1 + AddInputBias in one launch
+  ttmi_epilogue_args args{};
+  args.bias = dense_bias_2_.raw();
+  args.residual = input_tensor.raw();
+  TT_DEVICE_CALL(ttmi_gemm_fused(hidden_.raw(), packed2_.Get(dense_weight_2_, is_trans_weight), output->mutable_raw(), m, model_dim,
+                                 d_ff, d_ff, d_ff, model_dim, TTMI_EPI_BIAS_RESIDUAL, &args, kernels::DeviceDType(input_tensor),
+                                 Stream()));
+}
+
+void DistrillFFN::operator()(const Tensor& input_tensor, Tensor* output, bool is_trans_weight) const {
+  CheckFfn(input_tensor, dense_weight_1_, dense_bias_1_, dense_weight_2_, dense_bias_2_, is_trans_weight, "DistrillFFN");
+  const int64_t model_dim = input_tensor.shape(2), d_ff = PackedWeight::OutDim(dense_weight_1_, is_trans_weight);
+  const int64_t m = input_tensor.numel() / model_dim;
+  const DLDeviceType dev = input_tensor.device_type();
+  const int id = input_tensor.device_id();
+  hidden_.ReshapeAs(input_tensor.dtype(), {m, d_ff}, dev, id, "FFN/gemm0/Reshape");
+  GemmBiasAct(input_tensor, packed1_.Get(dense_weight_1_, is_trans_weight), d_ff, dense_bias_1_, TTMI_ACT_GELU, &hidden_);
+  output->ReshapeAs(input_tensor.dtype(), {input_tensor.shape(0), input_tensor.shape(1), model_dim}, dev, id, "FFN/Reshape");
+  // gemm1, then AddInputBias + LayerNorm as one AddBiasLayerNorm
+  GemmThenAddBiasLayerNorm(hidden_, packed2_.Get(dense_weight_2_, is_trans_weight), model_dim, dense_bias_2_, input_tensor,
+                           layer_norm_weight_, layer_norm_bias_, output);
+}
+
 void BertPooler::operator()(const Tensor& input_tensor, Tensor* output_tensor) const {
   kernels::RequireGpu(input_tensor, "BertPooler");
   TT_ENFORCE_EQ(input_tensor.shape(-1), dense_weight_.shape(0), "input width and weight rows differ");

@@ -86,6 +86,40 @@ class AlbertLayer {
   PackedWeight packed1_, packed2_;
 };
 
+// Feed-forward blocks of the decoder / DistilBERT wrappers (positionwise_ffn.h:23-84).  Weights are
+// [in, out], or [out, in] when called with is_trans_weight.
+class PositionwiseFeedForward {
+ public:
+  PositionwiseFeedForward(core::Tensor dense_weight_1, core::Tensor dense_bias_1, core::Tensor dense_weight_2,
+                          core::Tensor dense_bias_2, core::Tensor layer_norm_weight, core::Tensor layer_norm_bias)
+      : dense_weight_1_(std::move(dense_weight_1)), dense_bias_1_(std::move(dense_bias_1)),
+        dense_weight_2_(std::move(dense_weight_2)), dense_bias_2_(std::move(dense_bias_2)),
+        layer_norm_weight_(std::move(layer_norm_weight)), layer_norm_bias_(std::move(layer_norm_bias)) {}
+  // output = input + relu(LN(input) W1 + b1) W2 + b2, LayerNorm eps 1e-12   (positionwise_ffn.cpp:33-77)
+  void operator()(const core::Tensor& input_tensor, core::Tensor* output, bool is_trans_weight = false) const;
+
+ private:
+  core::Tensor dense_weight_1_, dense_bias_1_, dense_weight_2_, dense_bias_2_, layer_norm_weight_, layer_norm_bias_;
+  PackedWeight packed1_, packed2_;
+  mutable core::Tensor normed_, hidden_;
+};
+
+class DistrillFFN {
+ public:
+  DistrillFFN(core::Tensor dense_weight_1, core::Tensor dense_bias_1, core::Tensor dense_weight_2, core::Tensor dense_bias_2,
+              core::Tensor layer_norm_weight, core::Tensor layer_norm_bias)
+      : dense_weight_1_(std::move(dense_weight_1)), dense_bias_1_(std::move(dense_bias_1)),
+        dense_weight_2_(std::move(dense_weight_2)), dense_bias_2_(std::move(dense_bias_2)),
+        layer_norm_weight_(std::move(layer_norm_weight)), layer_norm_bias_(std::move(layer_norm_bias)) {}
+  // output = LN(input + gelu(input W1 + b1) W2 + b2), eps 1e-12   (positionwise_ffn.cpp:79-127)
+  void operator()(const core::Tensor& input_tensor, core::Tensor* output, bool is_trans_weight = false) const;
+
+ private:
+  core::Tensor dense_weight_1_, dense_bias_1_, dense_weight_2_, dense_bias_2_, layer_norm_weight_, layer_norm_bias_;
+  PackedWeight packed1_, packed2_;
+  mutable core::Tensor hidden_;
+};
+
 class PrepareBertMasks {
  public:
   // Fills missing position ids (0..S-1), token types (0) and mask (1), and builds the additive

@@ -183,6 +183,20 @@ PYBIND11_MODULE(turbo_transformers_cxx, m) {
       }))
       .def("__call__", &layers::AlbertLayer::operator());
 
+  py::class_<layers::PositionwiseFeedForward>(m, "PositionwiseFeedForward")
+      .def(py::init([](Tensor& w1, Tensor& b1, Tensor& w2, Tensor& b2, Tensor& ln_w, Tensor& ln_b) {
+        return new layers::PositionwiseFeedForward(std::move(w1), std::move(b1), std::move(w2), std::move(b2), std::move(ln_w),
+                                                   std::move(ln_b));
+      }))
+      .def("__call__", &layers::PositionwiseFeedForward::operator());
+
+  py::class_<layers::DistrillFFN>(m, "DistrillFFN")
+      .def(py::init([](Tensor& w1, Tensor& b1, Tensor& w2, Tensor& b2, Tensor& ln_w, Tensor& ln_b) {
+        return new layers::DistrillFFN(std::move(w1), std::move(b1), std::move(w2), std::move(b2), std::move(ln_w),
+                                       std::move(ln_b));
+      }))
+      .def("__call__", &layers::DistrillFFN::operator());
+
   py::class_<layers::FusedAddBiasGELU>(m, "FusedAddBiasGELU")
       .def(py::init([](Tensor& bias) { return new layers::FusedAddBiasGELU(std::move(bias)); }))
       .def("__call__", &layers::FusedAddBiasGELU::operator());

@@ -5,7 +5,7 @@ from .modeling_smart_pad import (MultiHeadedAttentionSmartBatch, BertLayerSmartB
 from .modeling_albert import (AlbertEmbeddings, AlbertAttention, AlbertLayer, AlbertLayerGroup, AlbertTransformer,
                               AlbertModel)
 from .qmodeling_bert import QBertIntermediate, QBertOutput, QBertAttention, QBertLayer, QBertEncoder, QBertModel
-from .modules import MultiHeadedAttention
+from .modules import MultiHeadedAttention, PositionwiseFeedForward, DistrillFFN
 from .return_type import ReturnType
 
 __all__ = [
@@ -13,5 +13,5 @@ __all__ = [
     'BertModelNoPooler', 'ReturnType', 'BertPooler', 'SequencePool', 'PoolingType', 'MultiHeadedAttentionSmartBatch',
     'BertLayerSmartBatch', 'BertEncoderSmartBatch', 'BertModelNoPoolerSmartBatch', 'BertModelSmartBatch',
     'QBertIntermediate', 'QBertOutput', 'QBertAttention', 'QBertLayer', 'QBertEncoder', 'QBertModel',
-    'MultiHeadedAttention', 'AlbertEmbeddings', 'AlbertAttention', 'AlbertLayer', 'AlbertLayerGroup', 'AlbertTransformer', 'AlbertModel',
+    'MultiHeadedAttention', 'PositionwiseFeedForward', 'DistrillFFN', 'AlbertEmbeddings', 'AlbertAttention', 'AlbertLayer', 'AlbertLayerGroup', 'AlbertTransformer', 'AlbertModel',
 ]

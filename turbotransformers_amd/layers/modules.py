@@ -15,7 +15,7 @@ from .return_type import ReturnType, convert_returns_as_type
 from .utils import (AnyTensor, convert2tt_tensor, create_empty_if_none, to_param_dict, try_convert, use_current_stream,
                     weight_in_out)
 
-__all__ = ['MultiHeadedAttention']
+__all__ = ['MultiHeadedAttention', 'PositionwiseFeedForward', 'DistrillFFN']
 
 
 class MultiHeadedAttention(cxx.MultiHeadedAttention):
@@ -78,3 +78,39 @@ class MultiHeadedAttention(cxx.MultiHeadedAttention):
             'weight': p['output.LayerNorm.weight'], 'bias': p['output.LayerNorm.bias']}
         args += [ln['weight'].detach().contiguous(), ln['bias'].detach().contiguous()]
         return MultiHeadedAttention(*[convert2tt_tensor(a) for a in args], attention.self.num_attention_heads)
+
+
+class _FeedForward:
+    """Shared call convention of the two feed-forward blocks (modules.py:233-290 of the reference)."""
+
+    def __call__(self, input_tensor: AnyTensor, return_type: Optional[ReturnType] = None, is_trans_weight: bool = False,
+                 output: Optional[cxx.Tensor] = None):
+        use_current_stream()
+        output = create_empty_if_none(output)
+        super().__call__(try_convert(input_tensor), output, is_trans_weight)
+        return convert_returns_as_type(output, return_type)
+
+    @classmethod
+    def _from_parts(cls, lin1, lin2, layer_norm, is_trans_weight):
+        pack = (lambda w: w.detach().contiguous()) if is_trans_weight else weight_in_out
+        with torch.no_grad():
+            args = [pack(lin1.weight), lin1.bias.detach().contiguous(), pack(lin2.weight), lin2.bias.detach().contiguous(),
+                    layer_norm.weight.detach().contiguous(), layer_norm.bias.detach().contiguous()]
+        return cls(*[convert2tt_tensor(a) for a in args])
+
+
+class PositionwiseFeedForward(_FeedForward, cxx.PositionwiseFeedForward):
+    """output = x + W2 relu(W1 LayerNorm(x) + b1) + b2 (OpenNMT-py's PositionwiseFeedForward)."""
+
+    @staticmethod
+    def from_onmt(position_wise_ffn, is_trans_weight: bool = False):
+        return PositionwiseFeedForward._from_parts(position_wise_ffn.w_1, position_wise_ffn.w_2, position_wise_ffn.layer_norm,
+                                                   is_trans_weight)
+
+
+class DistrillFFN(_FeedForward, cxx.DistrillFFN):
+    """output = LayerNorm(x + W2 gelu(W1 x + b1) + b2) (the feed-forward half of a DistilBERT block)."""
+
+    @staticmethod
+    def from_torch(ffn, layer_norm, is_trans_weight: bool = False):
+        return DistrillFFN._from_parts(ffn.lin1, ffn.lin2, layer_norm, is_trans_weight)

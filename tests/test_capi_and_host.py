@@ -47,11 +47,14 @@ def test_dropin_package_surface():
     import turbo_transformers.turbo_transformers_cxx as cxx
     for name in ("BertModel", "BertLayer", "BertEncoder", "BertAttention", "BertIntermediate", "BertOutput",
                  "BertEmbeddings", "BertPooler", "SequencePool", "PoolingType", "ReturnType", "BertModelSmartBatch",
-                 "MultiHeadedAttentionSmartBatch", "AlbertModel", "AlbertLayer"):
+                 "MultiHeadedAttentionSmartBatch", "AlbertModel", "AlbertLayer", "MultiHeadedAttention",
+                 "PositionwiseFeedForward", "DistrillFFN", "QBertModel", "pref_guard", "nparray2tensor", "tensor2nparrayf",
+                 "tensor2nparrayl", "enable_perf", "disable_perf", "set_num_threads", "reset_allocator_schema",
+                 "bert_opt_mem_allocate_api"):
         assert hasattr(tt, name), name
     for name in ("Tensor", "BERTEmbedding", "BertAttention", "MultiHeadedAttention", "MultiHeadedAttentionSmartBatch",
                  "BertIntermediate", "BertOutput", "SequencePool", "BertPooler", "PrepareBertMasks", "AlbertLayer",
-                 "FusedAddBiasGELU", "FusedAddBiasLayerNorm", "nparray2tensor", "tensor2nparrayf", "tensor2nparrayl",
+                 "FusedAddBiasGELU", "FusedAddBiasLayerNorm", "PositionwiseFeedForward", "DistrillFFN", "nparray2tensor", "tensor2nparrayf", "tensor2nparrayl",
                  "set_num_threads", "reset_allocator_schema", "bert_opt_mem_allocate_api", "enable_perf", "disable_perf",
                  "set_stderr_verbose_level"):
         assert hasattr(cxx, name), name

@@ -23,6 +23,25 @@ set_num_threads = cxx.set_num_threads
 reset_allocator_schema = cxx.reset_allocator_schema
 bert_opt_mem_allocate_api = cxx.bert_opt_mem_allocate_api
 set_stderr_verbose_level = cxx.set_stderr_verbose_level
+# python/turbo_transformers/utils.py:20-60 of the reference
+enable_perf = cxx.enable_perf
+disable_perf = cxx.disable_perf
+nparray2tensor = cxx.nparray2tensor
+tensor2nparrayf = cxx.tensor2nparrayf
+tensor2nparrayl = cxx.tensor2nparrayl
+
+import contextlib as _contextlib  # noqa: E402
+
+
+@_contextlib.contextmanager
+def pref_guard(filename: str):
+    """The reference's profiling scope.  Its gperftools profiler is not part of this build (rocprofv3 is the
+    tool here), so enable_perf / disable_perf are accepted and do nothing."""
+    cxx.enable_perf(filename)
+    yield
+    cxx.disable_perf()
+
 
 __all__ = list(_layers_all) + ['cxx', 'config', 'set_num_threads', 'reset_allocator_schema',
-                                'bert_opt_mem_allocate_api', 'set_stderr_verbose_level']
+                                'bert_opt_mem_allocate_api', 'set_stderr_verbose_level', 'enable_perf', 'disable_perf',
+                                'nparray2tensor', 'tensor2nparrayf', 'tensor2nparrayl', 'pref_guard']

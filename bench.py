@@ -129,6 +129,35 @@ MEASURED_TRAFFIC = {
 COPY_ELEMS = 64 << 20  # fp32 elements of the calibration copy: reads 256 MiB, writes 256 MiB
 
 
+def run_albert(steps, warmup):
+    """ALBERT: embedding size 128 projected to 768, one shared layer applied 12 times; fp16, batch 8 x seq 256."""
+    import torch
+    import turbo_transformers
+    from transformers import AlbertConfig, AlbertModel
+    torch.manual_seed(1234)
+    cfg = AlbertConfig(embedding_size=128, hidden_size=768, num_hidden_layers=12, num_attention_heads=12, intermediate_size=3072)
+    model = AlbertModel(cfg).eval().half().cuda()
+    tmodel = turbo_transformers.AlbertModel.from_torch(model)
+    ids = torch.randint(0, cfg.vocab_size, (8, 256), generator=torch.Generator().manual_seed(0)).cuda()
+    ms, p50, _, _ = time_steps(lambda: tmodel(ids), steps, warmup)
+    return {"ms_per_step": ms, "p50_ms": p50, "seq_per_s": 8 / ms * 1e3}
+
+
+def run_int8(steps, warmup):
+    """BERT-base with every Linear as int8 x int8 -> int32 (dynamic per-tensor activation scale, per-channel weight
+    scales), fp32 softmax / LayerNorm; batch 20 x seq 128."""
+    import torch
+    import turbo_transformers
+    from transformers import BertConfig, BertModel
+    torch.manual_seed(1234)
+    cfg = BertConfig()
+    model = BertModel(cfg).eval().cuda()
+    qmodel = turbo_transformers.QBertModel.from_torch(model, backend="turbo")
+    ids = torch.randint(0, cfg.vocab_size, (20, 128), generator=torch.Generator().manual_seed(0)).cuda()
+    ms, p50, _, _ = time_steps(lambda: qmodel(ids), steps, warmup)
+    return {"ms_per_step": ms, "p50_ms": p50, "seq_per_s": 20 / ms * 1e3}
+
+
 def kernel_rooflines(dtype="f16", batch=64, seq=512, hidden=768, heads=12, ffn=3072, iters=20, only=None):
     """Each kernel of the layer alone, at its real shape, timed with HIP events on the work stream
     through the C ABI.  GEMMs: algorithmic FLOPs = 2*M*N*K against the MFMA peak; memory-bound
@@ -363,6 +392,10 @@ def main():
                 r = run_dense(name, max(20, args.steps), args.warmup)
                 extras[name] = {k: r[k] for k in ("ms_per_step", "p50_ms", "seq_per_s", "host_wall_ms_per_step")}
         extras["smart_batch"] = run_smart_batch(max(10, args.steps // 2), args.warmup)
+        r = run_dense("large_bf16_b64_s512", 10, 2)
+        extras["large_bf16_b64_s512"] = {k: r[k] for k in ("ms_per_step", "p50_ms", "seq_per_s", "tflops")}
+        extras["albert_f16_b8_s256"] = run_albert(30, args.warmup)
+        extras["base_int8_b20_s128"] = run_int8(30, args.warmup)
         line["other_workloads"] = extras
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()

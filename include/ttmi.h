@@ -222,7 +222,9 @@ TTMI_API int ttmi_convert(const void* src, int src_dtype, void* dst, int dst_dty
 
 /* kernels::MatMul  (layers/kernels/mat_mul.cpp:30-118).
  * C[M,N] = alpha * A[M,K] * op(B) + beta * C, all row-major with leading dimensions in
- * elements.  trans_b = 0: B is [K,N] (ldb >= N);  trans_b != 0: B is [N,K] (ldb >= K). */
+ * elements.  trans_b = 0: B is [K,N] (ldb >= N);  trans_b != 0: B is [N,K] (ldb >= K).
+ * Problems with few output tiles and a long K run as K slices plus a reduction kernel; their fp32
+ * partial tiles live in a per-stream workspace this library allocates on first use and keeps. */
 TTMI_API int ttmi_gemm(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int64_t lda,
                        int64_t ldb, int64_t ldc, int trans_b, float alpha, float beta, int dtype,
                        void* stream);

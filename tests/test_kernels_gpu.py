@@ -295,3 +295,24 @@ def test_memcpy_and_memset(ttmi):
     assert np.array_equal(a, back)
     ok(ttmi.ttmi_memset_zero(ptr(d), a.nbytes, stream()))
     assert not host(d).any()
+
+
+def test_empty_inputs_are_accepted_and_touch_nothing(ttmi):
+    """Zero rows / zero tokens / zero batch: every entry point returns success without launching over
+    nothing, and a guard word behind each output stays untouched."""
+    guard = torch.full((64,), 3.0, device="cuda")
+    g, b = torch.ones(64, device="cuda"), torch.zeros(64, device="cuda")
+    ids = torch.zeros(1, dtype=torch.int64, device="cuda")
+    s = stream()
+    ok(ttmi.ttmi_layer_norm(ptr(guard), ptr(g), ptr(b), 0, 64, 1e-12, 0, s))
+    ok(ttmi.ttmi_add_bias_layer_norm(ptr(guard), ptr(guard), ptr(b), ptr(g), ptr(b), 0, 64, 1e-12, 0, s))
+    ok(ttmi.ttmi_add_bias_act(ptr(guard), ptr(b), 0, 64, 0, 0, s))
+    ok(ttmi.ttmi_apply_mask_and_softmax(ptr(guard), None, 0, 4, 8, 8, 1, 1.0, 0, s))
+    ok(ttmi.ttmi_transpose_for_score(ptr(g), ptr(guard), 0, 4, 2, 8, 0, s))
+    ok(ttmi.ttmi_lookup_embedding(ptr(guard), ptr(g), ptr(ids), 0, 64, 1, 0, 0, s))
+    ok(ttmi.ttmi_gemm(ptr(g), ptr(g), ptr(guard), 0, 8, 8, 8, 8, 8, 1, 1.0, 0.0, 0, s))
+    ok(ttmi.ttmi_gemm(ptr(g), ptr(g), ptr(guard), 8, 0, 8, 8, 8, 8, 1, 1.0, 0.0, 0, s))
+    ok(ttmi.ttmi_concat(ptr(g), ptr(g), ptr(guard), 0, 4, 4, 0, s))
+    ok(ttmi.ttmi_convert(ptr(g), 0, ptr(guard), 0, 0, s))
+    torch.cuda.synchronize()
+    assert bool((guard == 3.0).all())

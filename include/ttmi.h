@@ -114,6 +114,19 @@ TTMI_API int ttmi_add_bias_layer_norm_residual32(void* out, const float* residua
                                                  const void* gamma, const void* beta, float* out_f32, int64_t m,
                                                  int64_t n, float eps, int dtype, void* stream);
 
+/* The dense projection and AddBiasLayerNorm that close both halves of an encoder layer, as one call:
+ *   out[m,n] = LN(a[m,k] . w[n,k]^T + bias + residual)
+ * (BertOutput, layers/bert_output.cpp:41-60; the attention output, layers/multi_headed_attention.cpp:359-371;
+ * the reference issues MatMul then AddBiasLayerNorm).  Small problems, where the product is cut along K to
+ * fill the chip, normalise inside the kernel that sums the K slices; larger ones run ttmi_gemm followed by
+ * ttmi_add_bias_layer_norm.  Either `residual` (same dtype as out) or the pair residual_f32 / out_f32 (the
+ * fp32 residual stream of ttmi_add_bias_layer_norm_residual32, which may alias each other) is given; the
+ * unused ones are NULL.  a, w, out are densely packed (lda = ldb = k, ldc = n). */
+TTMI_API int ttmi_gemm_bias_layer_norm(const void* a, const void* w, void* out, const void* residual,
+                                       const float* residual_f32, const void* bias, const void* gamma,
+                                       const void* beta, float* out_f32, int64_t m, int64_t n, int64_t k, float eps,
+                                       int dtype, void* stream);
+
 /* kernels::AddBiasAct<T, Act>  (layers/kernels/activation.cpp:33-55, 90-119).
  * out[m,n] = act(out[m,n] + bias[n]) in place; gelu is the tanh form. */
 TTMI_API int ttmi_add_bias_act(void* out, const void* bias, int64_t m, int64_t n, int act, int dtype,

@@ -88,6 +88,70 @@ def test_fused_epilogues_small_m_long_k(ttmi, oracle, dt):
     assert max_abs(host(C), base + rounded(bias, dt) + rounded(res, dt)) <= GEMM_TOL[dt] * 3
 
 
+LN_TOL = {"f32": 1e-4, "f16": 4e-3, "bf16": 3e-2}  # relative to 1 + |expected|; large shapes round the product to 16 bits first
+
+
+def _ln_close(got, want, dt):
+    return bool(np.all(np.abs(got - want) <= LN_TOL[dt] * (1.0 + np.abs(want))))
+
+
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("M,N,K", [(128, 768, 768), (128, 768, 3072), (1, 768, 3072), (2560, 768, 3072), (300, 1024, 4096),
+                                   (40, 2052, 1024), (64, 4096, 1024), (64, 520, 256), (4096, 768, 768), (50, 770, 768)])
+def test_gemm_bias_layer_norm(ttmi, oracle, dt, M, N, K):
+    """Dense projection + AddBiasLayerNorm as one call: shapes that take the split-K kernels (normalised by
+    the kernel that sums the slices), and shapes that run the two kernels one after the other."""
+    rng = np.random.default_rng(M + N + K)
+    A, W = _ab(rng, M, N, K, 1)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    bias, gamma, beta = (rng.standard_normal(N).astype(np.float32) for _ in range(3))
+    dA, dW, dres = dev(A, dt), dev(W, dt), dev(res, dt)
+    out = torch.empty((M, N), dtype=dA.dtype, device="cuda")
+    out2 = torch.empty_like(out)
+    for o in (out, out2):
+        ok(ttmi.ttmi_gemm_bias_layer_norm(ptr(dA), ptr(dW), ptr(o), ptr(dres), None, ptr(dev(bias, dt)), ptr(dev(gamma, dt)),
+                                          ptr(dev(beta, dt)), None, M, N, K, 1e-12, TTMI_DTYPES[dt], stream()))
+    base = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    want = oracle.add_bias_layer_norm(base, rounded(res, dt), rounded(bias, dt), rounded(gamma, dt), rounded(beta, dt))
+    assert _ln_close(host(out), want, dt)
+    assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(128, 768, 3072), (2560, 1024, 4096), (4096, 768, 768)])
+def test_gemm_bias_layer_norm_fp32_residual(ttmi, oracle, dt, M, N, K):
+    """The same with the residual stream in fp32: the 16-bit output is the rounding of the fp32 one, and
+    writing the fp32 result over the residual buffer is allowed."""
+    rng = np.random.default_rng(M + N + K + 1)
+    A, W = _ab(rng, M, N, K, 1)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    bias, gamma, beta = (rng.standard_normal(N).astype(np.float32) for _ in range(3))
+    dA, dW, dres = dev(A, dt), dev(W, dt), dev(res)
+    out = torch.empty((M, N), dtype=dA.dtype, device="cuda")
+    out32 = torch.empty((M, N), device="cuda")
+    args = (ptr(dev(bias, dt)), ptr(dev(gamma, dt)), ptr(dev(beta, dt)))
+    ok(ttmi.ttmi_gemm_bias_layer_norm(ptr(dA), ptr(dW), ptr(out), None, ptr(dres), *args, ptr(out32), M, N, K, 1e-12,
+                                      TTMI_DTYPES[dt], stream()))
+    base = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    want = oracle.add_bias_layer_norm(base, res, rounded(bias, dt), rounded(gamma, dt), rounded(beta, dt))
+    assert _ln_close(host(out32), want, dt)
+    assert np.array_equal(host(out), rounded(host(out32), dt))
+    first = out32.clone()
+    ok(ttmi.ttmi_gemm_bias_layer_norm(ptr(dA), ptr(dW), ptr(out), None, ptr(dres), *args, ptr(dres), M, N, K, 1e-12,
+                                      TTMI_DTYPES[dt], stream()))
+    assert torch.equal(dres, first)
+
+
+def test_gemm_bias_layer_norm_rejects_bad_arguments(ttmi):
+    x = torch.zeros((8, 8), device="cuda")
+    v = torch.zeros(8, device="cuda")
+    # no residual at all; fp32 residual without its output
+    assert ttmi.ttmi_gemm_bias_layer_norm(ptr(x), ptr(x), ptr(x), None, None, ptr(v), ptr(v), ptr(v), None, 8, 8, 8, 1e-12,
+                                          TTMI_DTYPES["f32"], stream()) != 0
+    assert ttmi.ttmi_gemm_bias_layer_norm(ptr(x), ptr(x), ptr(x), None, ptr(x), ptr(v), ptr(v), ptr(v), None, 8, 8, 8, 1e-12,
+                                          TTMI_DTYPES["f32"], stream()) != 0
+
+
 @pytest.mark.parametrize("dt", ALL_DTYPES)
 def test_matmul_alpha_beta_and_ld(ttmi, oracle, dt):
     rng = np.random.default_rng(5)

@@ -681,6 +681,80 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   epi.store8(0, row, ncol, v, valid);
 }
 
+// The reduction of a split-K GEMM that feeds AddBiasLayerNorm, with the normalisation folded in:
+// one workgroup per output row sums the slices (fixed order), adds bias and residual, keeps the row in
+// registers (ITERS float4 per thread), and writes LN(x) -- one launch and one pass over the row
+// instead of a reduce kernel, a 16-bit round trip and a LayerNorm kernel.  Needs n % 4 == 0,
+// n <= 1024 * ITERS and rows of every operand aligned to four elements.   mean / variance as in layer_norm.cpp:144-163 of the reference.
+template <typename T, int ITERS>
+__global__ __launch_bounds__(256) void splitk_reduce_layer_norm_kernel(const float* __restrict__ ws, int splits, int m, int n,
+                                                                      const T* __restrict__ bias, const T* residual,
+                                                                      const float* residual32, const T* __restrict__ gamma,
+                                                                      const T* __restrict__ beta, T* out, float* out32, float eps) {
+  __shared__ float red[2][4];
+  const int row = blockIdx.x;
+  const int64_t mn = (int64_t)m * n;
+  float x[ITERS][4];
+  float sum = 0.f, sumsq = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int col = (it * 256 + threadIdx.x) * 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) x[it][j] = 0.f;
+    if (col < n) {
+      const float* p = ws + (int64_t)row * n + col;
+      for (int sidx = 0; sidx < splits; ++sidx) {
+        const float4 v = *reinterpret_cast<const float4*>(p + sidx * mn);
+        x[it][0] += v.x; x[it][1] += v.y; x[it][2] += v.z; x[it][3] += v.w;
+      }
+      const Vec<T, 4> b = load_vec<T, 4>(bias + col);
+      float r[4];
+      if (residual32 != nullptr) {
+        const float4 v = *reinterpret_cast<const float4*>(residual32 + (int64_t)row * n + col);
+        r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+      } else {
+        const Vec<T, 4> v = load_vec<T, 4>(residual + (int64_t)row * n + col);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = to_float(v.v[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[it][j] += to_float(b.v[j]) + r[j];
+        sum += x[it][j];
+        sumsq += x[it][j] * x[it][j];
+      }
+    }
+  }
+  sum = group_sum<kWave>(sum);
+  sumsq = group_sum<kWave>(sumsq);
+  if (threadIdx.x % kWave == 0) {
+    red[0][threadIdx.x / kWave] = sum;
+    red[1][threadIdx.x / kWave] = sumsq;
+  }
+  __syncthreads();
+  sum = red[0][0] + red[0][1] + red[0][2] + red[0][3];
+  sumsq = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+  const float mean = sum / (float)n;
+  const float var = sumsq / (float)n - mean * mean;
+  const float rstd = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int col = (it * 256 + threadIdx.x) * 4;
+    if (col < n) {
+      const Vec<T, 4> gm = load_vec<T, 4>(gamma + col), bt = load_vec<T, 4>(beta + col);
+      Vec<T, 4> o;
+      float y[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        y[j] = to_float(bt.v[j]) + to_float(gm.v[j]) * rstd * (x[it][j] - mean);
+        o.v[j] = from_float<T>(y[j]);
+      }
+      store_vec<T, 4>(out + (int64_t)row * n + col, o);
+      if (out32 != nullptr) *reinterpret_cast<float4*>(out32 + (int64_t)row * n + col) = make_float4(y[0], y[1], y[2], y[3]);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ fast-path kernel -----
 // Same tiling, for the shapes the encoder actually runs (B given as [N,K], 16-byte aligned
 // operands, K a multiple of the 128-byte K step).  Two differences from the general kernel:
@@ -979,8 +1053,9 @@ static int pick_splits(int64_t m, int64_t n, int64_t ksteps, int64_t batch) {
   return (int)std::max<int64_t>(1, std::min<int64_t>({(int64_t)compute_units() / tiles, ksteps / 4, 16}));
 }
 
-template <typename T, typename Epi>
-static int launch_splitk(GemmArgs g, const Epi& epi, int splits, int64_t ksteps, int bk, hipStream_t s) {
+// `reduce(ws, slices, vec, stream)` launches the kernel that sums the slices and applies the epilogue.
+template <typename T, typename Reduce>
+static int launch_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStream_t s, const Reduce& reduce) {
   const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
   float* ws = splitk_workspace(bytes, s);
   TTMI_REQUIRE(ws != nullptr, "cannot allocate the split-K workspace");
@@ -995,15 +1070,14 @@ static int launch_splitk(GemmArgs g, const Epi& epi, int splits, int64_t ksteps,
   const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
   hipLaunchKernelGGL((gemm_kernel<T, 64, 64, 2, 2, false, true, 2, EpiPartial>), dim3(grid_x, (unsigned)used, 1), dim3(256), LDS, s,
                      g, part);
-  const int64_t items = (int64_t)g.m * ((g.n + 7) / 8);
-  hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3((unsigned)ceil_div(items, 256)), dim3(256), 0, s, ws, used, g.m, g.n, vec, epi);
+  reduce(ws, used, vec, s);
   return launch_status("gemm_splitk");
 }
 
 // Split-K on the DMA kernel with 128x128 tiles, for mid-size problems whose tiles do not fill the chip
 // (M = 2560, N = 768, K = 3072: 120 tiles, 48 K steps each).
-template <typename T, typename Epi>
-static int launch_fast_splitk(GemmArgs g, const Epi& epi, int splits, int64_t ksteps, int bk, hipStream_t s) {
+template <typename T, typename Reduce>
+static int launch_fast_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStream_t s, const Reduce& reduce) {
   const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
   float* ws = splitk_workspace(bytes, s);
   TTMI_REQUIRE(ws != nullptr, "cannot allocate the split-K workspace");
@@ -1024,10 +1098,20 @@ static int launch_fast_splitk(GemmArgs g, const Epi& epi, int splits, int64_t ks
   // one workgroup per (tile, slice): the persistent loop runs once
   const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
   hipLaunchKernelGGL(kern, dim3(grid_x, (unsigned)used, 1), dim3(256), LDS, s, g, part);
-  const int64_t items = (int64_t)g.m * ((g.n + 7) / 8);
-  hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3((unsigned)ceil_div(items, 256)), dim3(256), 0, s, ws, used, g.m, g.n, vec, epi);
+  reduce(ws, used, vec, s);
   return launch_status("gemm_fast_splitk");
 }
+
+// The ordinary reduction: sum the slices, then the epilogue the unsplit kernel would have applied.
+template <typename Epi>
+struct ReduceWithEpilogue {
+  Epi epi;
+  int m, n;
+  void operator()(const float* ws, int slices, bool vec, hipStream_t s) const {
+    const int64_t items = (int64_t)m * ((n + 7) / 8);
+    hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3((unsigned)ceil_div(items, 256)), dim3(256), 0, s, ws, slices, m, n, vec, epi);
+  }
+};
 
 // Tile configurations of the fast path and a cost model to pick one.  With t = tile area /
 // efficiency as the time of one tile on an otherwise idle CU, and `per_cu` workgroups of that
@@ -1063,6 +1147,31 @@ static int pick_tile(int64_t m, int64_t n, int64_t batch) {
   return best;
 }
 
+// Whether (and how) a problem on the [N,K]-weights path is cut along K.
+enum class SplitKind { kNone, kSmallTiles, kDmaTiles };
+struct SplitPlan {
+  SplitKind kind;
+  int splits;
+};
+template <typename T>
+static SplitPlan plan_split(int64_t m, int64_t n, int64_t k, int64_t batch, bool aligned) {
+  constexpr int BK = kRowBytes / sizeof(T);
+  if (!aligned || k % BK != 0 || batch != 1) return {SplitKind::kNone, 1};
+  const int64_t ksteps = k / BK;
+  const int tile = pick_tile(m, n, batch);
+  if (tile == 3) {
+    const int64_t t128 = ceil_div(m, 128) * ceil_div(n, 128);
+    if (t128 <= compute_units() / 2 && ksteps >= 16) {
+      const int splits = (int)std::min<int64_t>({2 * (int64_t)compute_units() / t128, ksteps / 8, 8});
+      if (splits > 1) return {SplitKind::kDmaTiles, splits};
+    }
+  } else if (tile == 4) {
+    const int splits = pick_splits(m, n, ksteps, batch);
+    if (splits > 1) return {SplitKind::kSmallTiles, splits};
+  }
+  return {SplitKind::kNone, 1};
+}
+
 template <typename T, bool B_KN, typename Epi>
 static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipStream_t s) {
   if (g.m <= 0 || g.n <= 0 || batch <= 0) return 0;
@@ -1071,19 +1180,17 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
   if (!B_KN) {
     constexpr int BK = kRowBytes / sizeof(T);
     if (aligned && g.k % BK == 0) {
+      bool column_pass = false;
+      if constexpr (HasColumnPass<Epi>::value) column_pass = epi.v_pitch > 0;
       switch (pick_tile(g.m, g.n, batch)) {
         case 0: return launch_fast<T, 256, 256, 2, 4, Epi>(g, epi, batch, s);
         case 1: return launch_fast<T, 256, 192, 4, 2, Epi>(g, epi, batch, s);
         case 2: return launch_fast<T, 256, 128, 4, 2, Epi>(g, epi, batch, s);
         case 3: {
           if constexpr (std::is_same<typename Epi::Acc, float>::value) {
-            bool column_pass = false;
-            if constexpr (HasColumnPass<Epi>::value) column_pass = epi.v_pitch > 0;
-            const int64_t ksteps = g.k / BK, t128 = tiles(128, 128);
-            if (!column_pass && batch == 1 && t128 <= compute_units() / 2 && ksteps >= 16) {
-              const int splits = (int)std::min<int64_t>({2 * (int64_t)compute_units() / t128, ksteps / 8, 8});
-              if (splits > 1) return launch_fast_splitk<T, Epi>(g, epi, splits, ksteps, BK, s);
-            }
+            const SplitPlan plan = column_pass ? SplitPlan{SplitKind::kNone, 1} : plan_split<T>(g.m, g.n, g.k, batch, aligned);
+            if (plan.kind == SplitKind::kDmaTiles)
+              return launch_fast_splitk<T>(g, plan.splits, g.k / BK, BK, s, ReduceWithEpilogue<Epi>{epi, g.m, g.n});
           }
           return launch_fast<T, 128, 128, 2, 2, Epi>(g, epi, batch, s);
         }
@@ -1091,10 +1198,9 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
         // of a one-step prefetch better than the DMA path does with a tiny tile
         default: {
           if constexpr (std::is_same<typename Epi::Acc, float>::value) {
-            bool column_pass = false;
-            if constexpr (HasColumnPass<Epi>::value) column_pass = epi.v_pitch > 0;
-            const int splits = column_pass ? 1 : pick_splits(g.m, g.n, g.k / BK, batch);
-            if (splits > 1) return launch_splitk<T, Epi>(g, epi, splits, g.k / BK, BK, s);
+            const SplitPlan plan = column_pass ? SplitPlan{SplitKind::kNone, 1} : plan_split<T>(g.m, g.n, g.k, batch, aligned);
+            if (plan.kind == SplitKind::kSmallTiles)
+              return launch_splitk<T>(g, plan.splits, g.k / BK, BK, s, ReduceWithEpilogue<Epi>{epi, g.m, g.n});
           }
           return launch_config<T, 64, 64, 2, 2, false, true, Epi>(g, epi, batch, s);
         }
@@ -1254,6 +1360,54 @@ int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n,
     }
   });
   return 0;
+}
+
+int ttmi_gemm_bias_layer_norm(const void* a, const void* w, void* out, const void* residual, const float* residual_f32,
+                              const void* bias, const void* gamma, const void* beta, float* out_f32, int64_t m, int64_t n,
+                              int64_t k, float eps, int dtype, void* stream) {
+  TTMI_REQUIRE(a && w && out && bias && gamma && beta, "null tensor");
+  TTMI_REQUIRE((residual_f32 != nullptr) == (out_f32 != nullptr), "residual_f32 and out_f32 go together");
+  TTMI_REQUIRE(residual != nullptr || residual_f32 != nullptr, "a residual is required");
+  TTMI_REQUIRE(m >= 0 && n >= 0 && m < (1ll << 31) && n < (1ll << 31) && k < (1ll << 31), "dimension out of range");
+  if (m == 0 || n == 0) return 0;
+  TTMI_REQUIRE(k > 0, "K must be positive");
+  hipStream_t s = (hipStream_t)stream;
+  TTMI_DISPATCH_FLOAT(dtype, T, {
+    constexpr int KPC = 16 / sizeof(T);
+    const bool aligned = aligned16(a) && aligned16(w) && k % KPC == 0;
+    auto aligned_rows = [&](const void* p, size_t elem) { return (reinterpret_cast<uintptr_t>(p) % (4 * elem)) == 0; };
+    const bool rows_ok = n % 4 == 0 && n <= 4096 && aligned_rows(out, sizeof(T)) && aligned_rows(bias, sizeof(T)) &&
+                         aligned_rows(gamma, sizeof(T)) && aligned_rows(beta, sizeof(T)) &&
+                         (residual_f32 != nullptr ? aligned16(residual_f32) && aligned16(out_f32) : aligned_rows(residual, sizeof(T)));
+    const SplitPlan plan = rows_ok ? plan_split<T>(m, n, k, 1, aligned) : SplitPlan{SplitKind::kNone, 1};
+    if (plan.kind != SplitKind::kNone) {
+      GemmArgs g{};
+      g.a = (const char*)a;
+      g.b = (const char*)w;
+      g.m = (int)m; g.n = (int)n; g.k = (int)k;
+      g.lda = k; g.ldb = k;
+      g.inner = 1;
+      auto reduce = [&](const float* ws, int slices, bool, hipStream_t st) {
+        auto launch = [&](auto iters) {
+          hipLaunchKernelGGL((splitk_reduce_layer_norm_kernel<T, decltype(iters)::value>), dim3((unsigned)m), dim3(256), 0, st, ws,
+                             slices, (int)m, (int)n, (const T*)bias, (const T*)residual, residual_f32, (const T*)gamma,
+                             (const T*)beta, (T*)out, out_f32, eps);
+        };
+        if (n <= 1024) launch(std::integral_constant<int, 1>{});
+        else if (n <= 2048) launch(std::integral_constant<int, 2>{});
+        else launch(std::integral_constant<int, 4>{});
+      };
+      constexpr int BK = kRowBytes / sizeof(T);
+      if (plan.kind == SplitKind::kDmaTiles) return (launch_fast_splitk<T>(g, plan.splits, k / BK, BK, s, reduce));
+      return (launch_splitk<T>(g, plan.splits, k / BK, BK, s, reduce));
+    }
+  });
+  // Large problems: the GEMM kernel's own tiles cover the chip; LayerNorm follows as its own pass.
+  const int rc = ttmi_gemm(a, w, out, m, n, k, k, k, n, 1, 1.f, 0.f, dtype, stream);
+  if (rc != 0) return rc;
+  if (residual_f32 != nullptr)
+    return ttmi_add_bias_layer_norm_residual32(out, residual_f32, bias, gamma, beta, out_f32, m, n, eps, dtype, stream);
+  return ttmi_add_bias_layer_norm(out, residual, bias, gamma, beta, m, n, eps, dtype, stream);
 }
 
 int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_t n, int64_t k, int64_t lda,

@@ -59,9 +59,7 @@ static void GemmBiasAct(const Tensor& in, const void* w_nk, int64_t n, const Ten
 
 static void GemmThenAddBiasLayerNorm(const Tensor& in, const void* w_nk, int64_t n, const Tensor& bias, const Tensor& residual,
                                      const Tensor& gamma, const Tensor& beta, Tensor* out) {
-  const int64_t k = in.shape(-1), m = in.numel() / k;
-  TT_DEVICE_CALL(ttmi_gemm(in.raw(), w_nk, out->mutable_raw(), m, n, k, k, k, n, 1, 1.f, 0.f, kernels::DeviceDType(in), Stream()));
-  kernels::AddBiasLayerNormResidual(residual, bias, gamma, beta, out, 1e-12f);
+  kernels::GemmAddBiasLayerNorm(in, w_nk, n, residual, bias, gamma, beta, out, 1e-12f);
 }
 
 static std::vector<int64_t> WithLastDim(const Tensor& t, int64_t last) {

@@ -226,6 +226,36 @@ void AddBiasLayerNormResidual(const Tensor& input_tensor, const Tensor& bias_ten
                                                      DeviceDType(*out_tensor), Stream()));
 }
 
+void GemmAddBiasLayerNorm(const Tensor& in, const void* w_nk, int64_t n, const Tensor& residual, const Tensor& bias_tensor,
+                          const Tensor& gamma_tensor, const Tensor& beta_tensor, Tensor* out_tensor, float eps) {
+  RequireGpu(*out_tensor, "AddBiasLayerNorm");
+  const int64_t k = in.shape(-1), m = in.numel() / k;
+  TT_ENFORCE_EQ(n, gamma_tensor.shape(0), "AddBiasLayerNorm input_tensor.shape(-1) should be the same as gamma_tensor.shape(0)");
+  TT_ENFORCE_EQ(n, beta_tensor.shape(0), "AddBiasLayerNorm input_tensor.shape(-1) should be the same as beta_tensor.shape(0)");
+  TT_ENFORCE_EQ(n, bias_tensor.shape(0), "AddBiasLayerNorm input_tensor.shape(-1) should be the same as bias_tensor.shape(0)");
+  TT_ENFORCE_EQ(residual.numel(), m * n, "The shape of the input_tensor and out_tensor is not equal.");
+  TT_ENFORCE_EQ(out_tensor->numel(), m * n, "The shape of the input_tensor and out_tensor is not equal.");
+  const int dt = DeviceDType(*out_tensor);
+  if (!KeepsFp32Residual(*out_tensor)) {
+    TT_DEVICE_CALL(ttmi_gemm_bias_layer_norm(in.raw(), w_nk, out_tensor->mutable_raw(), residual.raw(), nullptr, bias_tensor.raw(),
+                                             gamma_tensor.raw(), beta_tensor.raw(), nullptr, m, n, k, eps, dt, Stream()));
+    return;
+  }
+  Tensor converted(nullptr);
+  const float* residual32 = nullptr;
+  if (residual.shadow() != nullptr) {
+    residual32 = residual.shadow()->data<float>();
+  } else {
+    float* p = converted.Reshape<float>({m, n}, residual.device_type(), residual.device_id(), "residual32");
+    TT_DEVICE_CALL(ttmi_convert(residual.raw(), DeviceDType(residual), p, TTMI_F32, m * n, Stream()));
+    residual32 = p;
+  }
+  Tensor* out32 = out_tensor->EnsureShadow();
+  TT_DEVICE_CALL(ttmi_gemm_bias_layer_norm(in.raw(), w_nk, out_tensor->mutable_raw(), nullptr, residual32, bias_tensor.raw(),
+                                           gamma_tensor.raw(), beta_tensor.raw(), out32->mutableData<float>(), m, n, k, eps, dt,
+                                           Stream()));
+}
+
 template <typename T, ActivationType ActType>
 void AddBiasAct(const Tensor& bias, Tensor* out, const std::string) {
   RequireGpu(*out, "AddBiasAct");

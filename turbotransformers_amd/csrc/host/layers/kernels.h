@@ -86,6 +86,11 @@ void AddBiasLayerNormResidual(const core::Tensor& input_tensor, const core::Tens
                               const core::Tensor& gamma_tensor, const core::Tensor& beta_tensor, core::Tensor* out_tensor,
                               float eps = 1e-12f);
 bool KeepsFp32Residual(const core::Tensor& t);  // true for bfloat16 tensors
+// out = AddBiasLayerNorm(in . w^T, residual) with the same treatment of the residual; `w_nk` is the
+// [n, k] weight on the device, `out_tensor` already has its [.., n] shape.
+void GemmAddBiasLayerNorm(const core::Tensor& in, const void* w_nk, int64_t n, const core::Tensor& residual,
+                          const core::Tensor& bias_tensor, const core::Tensor& gamma_tensor, const core::Tensor& beta_tensor,
+                          core::Tensor* out_tensor, float eps = 1e-12f);
 
 // ---- fused forms used by the layers (no counterpart in the reference's kernel API) --------
 int DeviceDType(const core::Tensor& t);  // ttmi_dtype of a floating tensor, throws otherwise

@@ -102,9 +102,7 @@ void MultiHeadedAttention::AttentionTail(const Tensor& query_tensor, const Tenso
   const void* wo = dense_packed_.Get(dense_weight_, is_trans_weight);
   if (!post_add_input && post_layernorm) {
     // gemm5 then AddBiasLayerNorm(query, bias, gamma, beta, out), eps 1e-12 (:359-371)
-    TT_DEVICE_CALL(ttmi_gemm(ctx_.raw(), wo, output->mutable_raw(), tokens, hidden, hidden, hidden, hidden, hidden, 1, 1.f, 0.f,
-                             dt, Stream()));
-    kernels::AddBiasLayerNormResidual(query_tensor, dense_bias_, layernorm_gamma_, layernorm_beta_, output, 1e-12f);
+    kernels::GemmAddBiasLayerNorm(ctx_, wo, hidden, query_tensor, dense_bias_, layernorm_gamma_, layernorm_beta_, output, 1e-12f);
   } else {
     ttmi_epilogue_args args{};
     args.bias = dense_bias_.raw();

@@ -31,7 +31,7 @@ extern "C" {
 #define TTMI_API __attribute__((visibility("default")))
 
 enum ttmi_dtype { TTMI_F32 = 0, TTMI_F16 = 1, TTMI_BF16 = 2, TTMI_I8 = 3, TTMI_I32 = 4, TTMI_I64 = 5 };
-enum ttmi_act { TTMI_ACT_GELU = 0, TTMI_ACT_TANH = 1, TTMI_ACT_RELU = 2 };
+enum ttmi_act { TTMI_ACT_NONE = -1, TTMI_ACT_GELU = 0, TTMI_ACT_TANH = 1, TTMI_ACT_RELU = 2 };
 enum ttmi_memcpy_kind { TTMI_H2D = 0, TTMI_D2H = 1, TTMI_D2D = 2 };
 enum ttmi_status {
   TTMI_OK = 0,
@@ -307,12 +307,15 @@ TTMI_API int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, i
 /* int8 path (quantized BERT: int8 x int8 -> int32 accumulators, exact).
  * ttmi_quantize_rows_i8: per-tensor symmetric dynamic scale from max|x| over the whole
  *   [m,k] activation: scale = max|x|/127 (1 if the tensor is all zero), q = clamp(rint(x/scale), -127, 127).
- *   `scale_dev` is a DEVICE float[2]: [0] receives the scale, [1] is scratch for the max.
+ *   `scale_dev` is a DEVICE float[TTMI_QUANT_SCALE_FLOATS]: [0] receives the scale, [1] max|x|, the rest is
+ *   scratch (per-workgroup maxima; nothing has to be cleared between calls).
  * ttmi_gemm_i8: C_i32[M,N] = A_i8[M,K] * B_i8[N,K]^T.
  * ttmi_dequant_bias: out[m,n] = acc[m,n] * (*act_scale) * w_scale[n] + bias[n] (fp32 out; bias may be NULL).
  * ttmi_gemm_i8_dequant: ttmi_gemm_i8 followed by ttmi_dequant_bias in one kernel (the accumulators never
- *   reach memory); same operation order, same bits.  Together they stand in for the dynamically
+ *   reach memory); same operation order, same bits.  `act` other than TTMI_ACT_NONE also applies that
+ *   activation, as ttmi_add_bias_act would after the bias (the FusedAddBiasGELU step of QBertIntermediate).  Together they stand in for the dynamically
  *   quantised Linear module the reference's QBert* layers call (qmodeling_bert.py:17,35). */
+#define TTMI_QUANT_SCALE_FLOATS 514
 /* ttmi_quantize_weight_rows_i8: per-output-channel symmetric scales for a weight w[N,K] (fp32):
  *   scales[n] = max_k |w[n,k]| / 127 (1 if the row is zero), q[n,k] = clamp(rint(w[n,k]/scales[n]), -127, 127). */
 TTMI_API int ttmi_quantize_weight_rows_i8(const float* w, int8_t* q, float* scales, int64_t n, int64_t k,
@@ -322,7 +325,7 @@ TTMI_API int ttmi_quantize_rows_i8(const float* x, int8_t* q, float* scale_dev, 
 TTMI_API int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_t n, int64_t k,
                           int64_t lda, int64_t ldb, int64_t ldc, void* stream);
 TTMI_API int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev,
-                                  const float* w_scale, const float* bias, int64_t m, int64_t n, int64_t k,
+                                  const float* w_scale, const float* bias, int act, int64_t m, int64_t n, int64_t k,
                                   int64_t lda, int64_t ldb, int64_t ldc, void* stream);
 TTMI_API int ttmi_dequant_bias(const int32_t* acc, const float* act_scale_dev, const float* w_scale,
                                const float* bias, float* out, int64_t m, int64_t n, void* stream);

@@ -361,11 +361,19 @@ def test_gemm_i8_dequant_equals_unfused(ttmi, oracle, M, N, K, with_bias):
     two_step, fused = torch.empty((M, N), device="cuda"), torch.empty((M, N), device="cuda")
     ok(ttmi.ttmi_gemm_i8(ptr(dA), ptr(dB), ptr(acc), M, N, K, K, K, N, stream()))
     ok(ttmi.ttmi_dequant_bias(ptr(acc), ptr(dsx), ptr(dsw), ptr(dbias) if with_bias else None, ptr(two_step), M, N, stream()))
-    ok(ttmi.ttmi_gemm_i8_dequant(ptr(dA), ptr(dB), ptr(fused), ptr(dsx), ptr(dsw), ptr(dbias) if with_bias else None, M, N, K, K,
-                                 K, N, stream()))
+    ok(ttmi.ttmi_gemm_i8_dequant(ptr(dA), ptr(dB), ptr(fused), ptr(dsx), ptr(dsw), ptr(dbias) if with_bias else None, -1, M, N,
+                                 K, K, K, N, stream()))
     assert np.array_equal(host(fused), host(two_step))
     want = oracle.dequant_bias(oracle.gemm_i8(a, b), sx[0], sw, bias if with_bias else np.zeros(N, np.float32))
     assert max_abs(host(fused), want) <= 1e-5 * max(1.0, float(np.abs(want).max()))
+    # with the activation folded in as well: the bits of the stand-alone bias + GELU kernel on the unbiased product
+    if with_bias:
+        ok(ttmi.ttmi_dequant_bias(ptr(acc), ptr(dsx), ptr(dsw), None, ptr(two_step), M, N, stream()))
+        ok(ttmi.ttmi_add_bias_act(ptr(two_step), ptr(dbias), M, N, capi.ACT_GELU, TTMI_DTYPES["f32"], stream()))
+        ok(ttmi.ttmi_gemm_i8_dequant(ptr(dA), ptr(dB), ptr(fused), ptr(dsx), ptr(dsw), ptr(dbias), capi.ACT_GELU, M, N, K, K, K,
+                                     N, stream()))
+        assert max_abs(host(fused), host(two_step)) <= 1e-6 * max(1.0, float(np.abs(want).max()))
+        assert max_abs(host(fused), oracle.add_bias_act(want, np.zeros(N, np.float32), 0)) <= 2e-5 * max(1.0, float(np.abs(want).max()))
 
 
 def test_int8_linear_pipeline(ttmi, oracle):
@@ -378,7 +386,7 @@ def test_int8_linear_pipeline(ttmi, oracle):
     qw, sw = oracle.quantize_weight_i8(w)
     qx_want, sx_want = oracle.quantize_tensor_i8(x)
     dq = torch.empty((M, K), dtype=torch.int8, device="cuda")
-    scale = torch.empty(2, device="cuda")
+    scale = torch.full((capi.QUANT_SCALE_FLOATS, ), float("nan"), device="cuda")  # scratch needs no clearing
     ok(ttmi.ttmi_quantize_rows_i8(ptr(dev(x)), ptr(dq), ptr(scale), M, K, stream()))
     assert np.array_equal(host(dq), qx_want)
     assert host(scale)[0] == np.float32(sx_want)

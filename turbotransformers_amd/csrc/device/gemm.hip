@@ -346,6 +346,7 @@ struct EpiDequant {
   const float* bias;       // [N] or null
   int64_t ldc;
   bool vec;
+  int act;  // ttmi_act, applied after the bias
   __device__ __forceinline__ const float* bias_ptr() const { return nullptr; }  // added after scaling, below
   __device__ __forceinline__ void store8(int, int m, int n, int (&v)[8], int valid) const {
     const float sx = act_scale[0];
@@ -357,6 +358,16 @@ struct EpiDequant {
         r[j] = (float)v[j] * sx * w_scale[n + j];
         if (bias) r[j] += bias[n + j];
       }
+    }
+    if (act == TTMI_ACT_GELU) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) r[j] = apply_act<TTMI_ACT_GELU>(r[j]);
+    } else if (act == TTMI_ACT_TANH) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) r[j] = apply_act<TTMI_ACT_TANH>(r[j]);
+    } else if (act == TTMI_ACT_RELU) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) r[j] = apply_act<TTMI_ACT_RELU>(r[j]);
     }
     float* p = c + (int64_t)m * ldc + n;
     if (vec && valid == 8) {
@@ -1427,9 +1438,10 @@ int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_
 }
 
 int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev, const float* w_scale,
-                         const float* bias, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc,
+                         const float* bias, int act, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc,
                          void* stream) {
   TTMI_REQUIRE(a && b && c && act_scale_dev && w_scale, "null tensor");
+  TTMI_REQUIRE(act >= TTMI_ACT_NONE && act <= TTMI_ACT_RELU, "unknown activation");
   TTMI_REQUIRE(m < (1ll << 31) && n < (1ll << 31) && k < (1ll << 31), "dimension too large");
   TTMI_REQUIRE(lda >= k && ldb >= k && ldc >= n, "leading dimension too small");
   GemmArgs g{};
@@ -1438,7 +1450,7 @@ int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float
   g.m = (int)m; g.n = (int)n; g.k = (int)k;
   g.lda = lda; g.ldb = ldb;
   g.inner = 1;
-  EpiDequant epi{c, act_scale_dev, w_scale, bias, ldc, aligned16(c) && ldc % 4 == 0};
+  EpiDequant epi{c, act_scale_dev, w_scale, bias, ldc, aligned16(c) && ldc % 4 == 0, act};
   const bool aligned = aligned16(a) && aligned16(b) && lda % 16 == 0 && ldb % 16 == 0 && k % 16 == 0;
   return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
 }

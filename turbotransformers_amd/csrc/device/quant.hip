@@ -4,10 +4,19 @@
 
 namespace ttmi {
 
-// |x| as uint bits orders like the float for non-negative values, so one integer
-// atomicMax per block yields max|x|.
-__global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ x, int64_t n,
-                                                     uint32_t* __restrict__ out_bits) {
+// max|x| in two steps without atomics or a cleared cell: every workgroup of absmax_kernel writes the
+// maximum of its share to partial[blockIdx.x]; every workgroup of quantize_kernel then reduces those (at
+// most kMaxPartials) values itself before it quantises its share.  Results do not depend on scheduling.
+constexpr int kMaxPartials = 512;
+
+__device__ __forceinline__ float block_max_256(float mx, float* red) {
+  mx = group_max<kWave>(mx);
+  if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = mx;
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+__global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ x, int64_t n, float* __restrict__ partial) {
   __shared__ float red[4];
   float mx = 0.f;
   int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
@@ -21,27 +30,41 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ x
     i += n4 * 4;
   }
   for (; i < n; i += stride) mx = fmaxf(mx, fabsf(x[i]));
-  mx = group_max<kWave>(mx);
-  if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = mx;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    atomicMax(out_bits, __float_as_uint(mx));
-  }
+  mx = block_max_256(mx, red);
+  if (threadIdx.x == 0) partial[blockIdx.x] = mx;
+}
+
+__device__ __forceinline__ int quantize_one(float x, float scale) {
+  float r = rintf(x / scale);  // round half to even
+  r = fminf(fmaxf(r, -127.f), 127.f);
+  return (int)r;
 }
 
 __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, int8_t* __restrict__ q,
-                                                       float* __restrict__ scale_dev, int64_t n) {
-  const float mx = scale_dev[1];
+                                                       float* __restrict__ scale_dev, int partials, int64_t n) {
+  __shared__ float red[4];
+  const float* partial = scale_dev + 2;
+  float mx = 0.f;
+  for (int p = threadIdx.x; p < partials; p += 256) mx = fmaxf(mx, partial[p]);
+  mx = block_max_256(mx, red);
   const float scale = mx > 0.f ? mx / 127.0f : 1.0f;
   int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
-  if (i == 0) scale_dev[0] = scale;
-  for (; i < n; i += stride) {
-    float r = rintf(x[i] / scale);  // round half to even
-    r = fminf(fmaxf(r, -127.f), 127.f);
-    q[i] = (int8_t)r;
+  if (i == 0) {
+    scale_dev[0] = scale;
+    scale_dev[1] = mx;
   }
+  if (((reinterpret_cast<uintptr_t>(x) & 15) | (reinterpret_cast<uintptr_t>(q) & 3)) == 0) {  // 4 elements per lane
+    const int64_t n4 = n / 4;
+    for (int64_t j = i; j < n4; j += stride) {
+      const float4 v = reinterpret_cast<const float4*>(x)[j];
+      const uint32_t packed = (uint32_t)(quantize_one(v.x, scale) & 255) | ((uint32_t)(quantize_one(v.y, scale) & 255) << 8) |
+                              ((uint32_t)(quantize_one(v.z, scale) & 255) << 16) | ((uint32_t)(quantize_one(v.w, scale) & 255) << 24);
+      reinterpret_cast<uint32_t*>(q)[j] = packed;
+    }
+    i += n4 * 4;
+  }
+  for (; i < n; i += stride) q[i] = (int8_t)quantize_one(x[i], scale);
 }
 
 __global__ __launch_bounds__(256) void dequant_bias_kernel(const int32_t* __restrict__ acc,
@@ -104,12 +127,11 @@ int ttmi_quantize_rows_i8(const float* x, int8_t* q, float* scale_dev, int64_t m
   const int64_t n = m * k;
   if (n <= 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  int rc = ttmi_memset_zero(scale_dev, 2 * sizeof(float), stream);
-  if (rc != 0) return rc;
-  // one atomic per workgroup on a single word: a few hundred workgroups keep that cheap
-  const unsigned absmax_grid = (unsigned)std::min<int64_t>(ceil_div(n, 256 * 16), 512);
-  hipLaunchKernelGGL(absmax_kernel, dim3(std::max(absmax_grid, 1u)), dim3(256), 0, s, x, n, reinterpret_cast<uint32_t*>(scale_dev + 1));
-  hipLaunchKernelGGL(quantize_kernel, dim3(flat_grid(n)), dim3(256), 0, s, x, q, scale_dev, n);
+  const int partials = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n, 256 * 16), kMaxPartials));
+  static_assert(kMaxPartials + 2 == TTMI_QUANT_SCALE_FLOATS, "scale_dev holds the scale, the maximum and the partial maxima");
+  hipLaunchKernelGGL(absmax_kernel, dim3((unsigned)partials), dim3(256), 0, s, x, n, scale_dev + 2);
+  const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(n, 256 * 4), 256 * 8);
+  hipLaunchKernelGGL(quantize_kernel, dim3(std::max(grid, 1u)), dim3(256), 0, s, x, q, scale_dev, partials, n);
   return launch_status("quantize_rows_i8");
 }
 

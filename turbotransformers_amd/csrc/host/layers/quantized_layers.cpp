@@ -14,6 +14,15 @@ using core::Tensor;
 
 static void* Stream() { return DeviceContext::GetInstance().stream(); }
 
+QuantizedLinear::QuantizedLinear(core::Tensor weight, core::Tensor bias, const std::string& activation)
+    : weight_(std::move(weight)), bias_(std::move(bias)) {
+  TT_ENFORCE_EQ(bias_.numel(), weight_.shape(1), "bias and weight shape mismatch");
+  if (activation == "gelu") act_ = TTMI_ACT_GELU;
+  else if (activation == "tanh") act_ = TTMI_ACT_TANH;
+  else if (activation == "relu") act_ = TTMI_ACT_RELU;
+  else TT_ENFORCE(activation.empty(), "unknown activation %s", activation.c_str());
+}
+
 void QuantizedLinear::Prepare() const {
   if (prepared_) return;
   kernels::RequireGpu(weight_, "QuantizedLinear");
@@ -27,7 +36,7 @@ void QuantizedLinear::Prepare() const {
   int8_t* q = q_weight_.Reshape<int8_t>({n, k}, dev, id, "QuantizedLinear/q_weight");
   float* s = w_scales_.Reshape<float>({n}, dev, id, "QuantizedLinear/w_scales");
   TT_DEVICE_CALL(ttmi_quantize_weight_rows_i8(t, q, s, n, k, Stream()));
-  act_scale_.Reshape<float>({2}, dev, id, "QuantizedLinear/act_scale");
+  act_scale_.Reshape<float>({TTMI_QUANT_SCALE_FLOATS}, dev, id, "QuantizedLinear/act_scale");
   prepared_ = true;
 }
 
@@ -47,8 +56,8 @@ void QuantizedLinear::operator()(const Tensor& input_tensor, Tensor* output_tens
   float* scale = act_scale_.mutableData<float>();
   TT_DEVICE_CALL(ttmi_quantize_rows_i8(input_tensor.data<float>(), qx, scale, m, k, Stream()));
   // int8 GEMM with the dequantisation folded into its store: the int32 accumulators stay on chip
-  TT_DEVICE_CALL(ttmi_gemm_i8_dequant(qx, q_weight_.data<int8_t>(), out, scale, w_scales_.data<float>(), nullptr, m, n, k, k, k,
-                                      n, Stream()));
+  TT_DEVICE_CALL(ttmi_gemm_i8_dequant(qx, q_weight_.data<int8_t>(), out, scale, w_scales_.data<float>(),
+                                      bias_.is_null() ? nullptr : bias_.data<float>(), act_, m, n, k, k, k, n, Stream()));
 }
 
 void QuantizedBertAttention::operator()(const Tensor& input_tensor, const Tensor& attention_mask, Tensor* output,

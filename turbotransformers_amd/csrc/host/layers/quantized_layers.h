@@ -6,11 +6,13 @@
 // In the reference the int8 GEMM is not C++ at all: QBertIntermediate / QBertOutput wrap
 // torch.quantization.quantize_dynamic modules (python/turbo_transformers/layers/qmodeling_bert.py:17,35)
 // and only the fused fp32 epilogues are turbo kernels.  The classes here keep that split
-// (QuantizedLinear has no bias; FusedAddBiasGELU / FusedAddBiasLayerNorm follow it) and add
-// QuantizedBertAttention so that every Linear of the layer is int8.
+// (QuantizedLinear alone has no bias; FusedAddBiasGELU / FusedAddBiasLayerNorm can follow it), let
+// QuantizedLinear take the bias and activation into its own kernel, and add QuantizedBertAttention so
+// that every Linear of the layer is int8.
 #pragma once
 
 #include <mutex>
+#include <string>
 
 #include "core/tensor.h"
 
@@ -20,15 +22,19 @@ namespace layers {
 class QuantizedLinear {
  public:
   // weight: fp32 [in, out] (the layout every other layer takes); quantized on first use.
-  explicit QuantizedLinear(core::Tensor weight) : weight_(std::move(weight)) {}
-  // output[tokens, out] (fp32) = dequant(q(input) * q(weight)^T); no bias.
+  explicit QuantizedLinear(core::Tensor weight) : weight_(std::move(weight)), bias_(nullptr) {}
+  // With a bias and an activation ("gelu", "tanh", "relu", or "" for none) applied by the same kernel that
+  // dequantises the product: Linear + FusedAddBiasGELU of QBertIntermediate as one call.
+  QuantizedLinear(core::Tensor weight, core::Tensor bias, const std::string& activation);
+  // output[tokens, out] (fp32) = act(dequant(q(input) * q(weight)^T) + bias)
   void operator()(const core::Tensor& input_tensor, core::Tensor* output_tensor) const;
   int64_t in_features() const { return weight_.shape(0); }
   int64_t out_features() const { return weight_.shape(1); }
 
  private:
   void Prepare() const;
-  core::Tensor weight_;
+  core::Tensor weight_, bias_;
+  int act_ = -1;  // ttmi_act; -1 = none
   mutable core::Tensor q_weight_, w_scales_, q_input_, acc_, act_scale_;
   mutable bool prepared_ = false;
 };

@@ -213,6 +213,9 @@ PYBIND11_MODULE(turbo_transformers_cxx, m) {
 
   py::class_<layers::QuantizedLinear>(m, "QuantizedLinear")
       .def(py::init([](Tensor& w) { return new layers::QuantizedLinear(std::move(w)); }))
+      .def(py::init([](Tensor& w, Tensor& bias, const std::string& activation) {
+        return new layers::QuantizedLinear(std::move(w), std::move(bias), activation);
+      }))
       .def("__call__", &layers::QuantizedLinear::operator());
 
   py::class_<layers::QuantizedBertAttention>(m, "QuantizedBertAttention")

@@ -23,14 +23,14 @@ __all__ = ['QBertIntermediate', 'QBertOutput', 'QBertAttention', 'QBertLayer', '
 class QBertIntermediate:
     def __init__(self, intermediate):
         p = to_param_dict(intermediate)
-        self.linear = cxx.QuantizedLinear(convert2tt_tensor(weight_in_out(p['dense.weight'])))
-        self.turbo_bias_act = cxx.FusedAddBiasGELU(convert2tt_tensor(p['dense.bias']))
+        # Linear and the reference's FusedAddBiasGELU step (qmodeling_bert.py:17-28) in one kernel
+        self.linear = cxx.QuantizedLinear(convert2tt_tensor(weight_in_out(p['dense.weight'])),
+                                          convert2tt_tensor(p['dense.bias']), "gelu")
 
     def __call__(self, input_tensor, return_type: Optional[ReturnType] = None):
         use_current_stream()
         out = cxx.Tensor.create_empty()
         self.linear(try_convert(input_tensor), out)
-        self.turbo_bias_act(out)
         return convert_returns_as_type(out, return_type)
 
     @staticmethod

@@ -1,0 +1,165 @@
+"""Parity at the full benchmark shapes: BERT-base fp16 and BERT-large bf16, batch 64 x seq 512 (32768 tokens).
+
+The CPU oracle needs about a second per 512-token sequence, so the full batch is checked (a) against
+the oracle on a sample of its sequences, and (b) through properties that hold at any size and that a
+mis-indexed tile, a dropped K step or a leaking pad column would break:
+  * the rows of one sequence do not depend on the rest of the batch (permuting the batch permutes the
+    output bit for bit; a sequence alone gives the rows it gives inside the batch),
+  * tokens under the padding mask do not influence valid rows (bit for bit),
+  * GEMM: column sums of A.W equal (1^T A).W, to the rounding of the stored outputs,
+  * attention: rows of softmax sum to one (V = 1 gives 1), and the one-kernel form agrees with the
+    four-kernel chain of the reference at the full shape,
+  * LayerNorm with gamma = 1, beta = 0: every row has mean 0 and variance 1.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import TTMI_DTYPES, dev, host, max_abs, ok, oracle_layer_weights, ptr, stream
+
+pytestmark = pytest.mark.gpu
+
+B, S, H, HEADS, FFN, LAYERS = 64, 512, 768, 12, 3072, 12
+# (name, layers, hidden, heads, ffn, dtype, sequences checked against the oracle)
+SHAPES = [("base_f16", LAYERS, H, HEADS, FFN, torch.float16, (0, 37, 63)),
+          ("large_bf16", 24, 1024, 16, 4096, torch.bfloat16, (63, ))]
+
+
+@pytest.fixture(scope="module", params=SHAPES, ids=[c[0] for c in SHAPES])
+def full(request):
+    """The 16-bit model, its weights as fp32 arrays for the oracle, ids and a mask with ragged tails, and the
+    output of one forward of the whole batch."""
+    import copy
+    import turbo_transformers as tt
+    from transformers import BertConfig, BertModel
+    _, layers, hidden, heads, ffn, dtype, sampled = request.param
+    torch.manual_seed(1234)
+    cfg = BertConfig(num_hidden_layers=layers, hidden_size=hidden, num_attention_heads=heads, intermediate_size=ffn,
+                     hidden_act="gelu_pytorch_tanh", hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0)
+    model = BertModel(cfg).eval()
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("bias") or "LayerNorm.weight" in name:
+                p.add_(0.05 * torch.randn_like(p))
+    low = copy.deepcopy(model).to(dtype).cuda()
+    weights = {k: v.detach().float().cpu().numpy() for k, v in low.named_parameters()}
+    rng = np.random.default_rng(0)
+    ids = rng.integers(0, cfg.vocab_size, (B, S))
+    lens = rng.integers(S // 4, S + 1, B)
+    lens[0], lens[63] = S, 200
+    mask = (np.arange(S)[None, :] < lens[:, None]).astype(np.int64)
+    tmodel = tt.BertModel.from_torch(low, torch.device("cuda:0"), "turbo")
+    d_ids, d_mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    out = tmodel(d_ids, attention_masks=d_mask)[0].clone()
+    yield {"model": tmodel, "weights": weights, "ids": ids, "mask": mask, "lens": lens, "d_ids": d_ids, "d_mask": d_mask,
+           "out": out, "layers": layers, "heads": heads, "dtype": dtype, "sampled": sampled}
+    del tmodel, low
+    torch.cuda.empty_cache()
+
+
+def test_sampled_sequences_of_the_full_batch_match_the_oracle(full, oracle):
+    w = full["weights"]
+    layers = [oracle_layer_weights(w, f"encoder.layer.{i}.") for i in range(full["layers"])]
+    got = host(full["out"])
+    for b in full["sampled"]:
+        ids, n = full["ids"][b:b + 1], int(full["lens"][b])
+        emb = oracle.bert_embedding(ids, np.arange(S)[None], np.zeros((1, S), np.int64), w["embeddings.word_embeddings.weight"],
+                                    w["embeddings.position_embeddings.weight"], w["embeddings.token_type_embeddings.weight"],
+                                    w["embeddings.LayerNorm.weight"], w["embeddings.LayerNorm.bias"])
+        ext = (-10000.0 * (1 - full["mask"][b])).astype(np.float32).reshape(1, 1, 1, S)
+        want = oracle.bert_encoder(emb, ext, layers, full["heads"])[0]
+        # rows under the mask are computed too (as the reference does) but nothing downstream reads them
+        err = np.abs(got[b, :n] - want[:n])
+        if full["dtype"] == torch.float16:
+            assert err.max() < 2e-2, "sequence %d" % b
+        else:
+            # a bfloat16 output carries half an ulp (2^-8 relative) of representation error whatever computed
+            # it; the bound applies to what exceeds that, as a quantile plus a cap over the 24 layers
+            excess = err - 2.0 ** -8 * np.abs(want[:n])
+            assert (excess > 2e-2).mean() <= 1e-4 and excess.max() < 3e-2, "sequence %d" % b
+
+
+def test_permuting_the_batch_permutes_the_output_bit_for_bit(full):
+    perm = torch.from_numpy(np.random.default_rng(1).permutation(B)).cuda()
+    out = full["model"](full["d_ids"][perm].contiguous(), attention_masks=full["d_mask"][perm].contiguous())[0]
+    assert torch.equal(out, full["out"][perm])
+
+
+def test_tokens_under_the_mask_do_not_reach_valid_rows(full):
+    ids = full["ids"].copy()
+    rng = np.random.default_rng(2)
+    pad = full["mask"] == 0
+    ids[pad] = rng.integers(0, 30522, int(pad.sum()))
+    out = full["model"](torch.from_numpy(ids).cuda(), attention_masks=full["d_mask"])[0]
+    valid = full["d_mask"].bool()
+    assert torch.equal(out[valid], full["out"][valid])
+    assert not torch.equal(out, full["out"])  # the pad rows themselves did change
+
+
+def test_a_sequence_alone_gives_its_rows_of_the_batch(full):
+    """Batch 1 takes other tile shapes (and the K-split kernels), so this is a tolerance, not bits."""
+    tol = 1e-2 if full["dtype"] == torch.float16 else 6e-2  # bf16: an ulp is 0.03 at |x| = 4
+    for b in (5, 63):
+        alone = full["model"](full["d_ids"][b:b + 1].contiguous(), attention_masks=full["d_mask"][b:b + 1].contiguous())[0]
+        n = int(full["lens"][b])
+        assert max_abs(host(alone)[0, :n], host(full["out"])[b, :n]) < tol
+
+
+@pytest.mark.parametrize("N,K", [(2304, 768), (768, 768), (3072, 768), (768, 3072)])
+def test_gemm_column_checksums_at_full_size(ttmi, N, K):
+    """sum_m C[m, n] = (sum_m A[m, :]) . W[n, :].  fp32 accumulation errs by ~K * 2^-24 relative; what
+    remains is the rounding of each stored output, at most half an ulp (2^-11 relative) each."""
+    M = B * S
+    g = torch.Generator(device="cuda").manual_seed(N + K)
+    A = torch.randn((M, K), generator=g, device="cuda").half()
+    W = (torch.randn((N, K), generator=g, device="cuda") / K ** 0.5).half()
+    C = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ok(ttmi.ttmi_gemm(ptr(A), ptr(W), ptr(C), M, N, K, K, K, N, 1, 1.0, 0.0, TTMI_DTYPES["f16"], stream()))
+    a_sum = host(A).astype(np.float64).sum(0)
+    want = host(W).astype(np.float64) @ a_sum
+    c = host(C).astype(np.float64)
+    bound = 2.0 ** -11 * np.abs(c).sum(0) * 1.05 + 1e-3
+    assert (np.abs(c.sum(0) - want) <= bound).all()
+    # and the same along the other axis: C . 1 = A . (W^T 1)
+    want_rows = host(A).astype(np.float64) @ host(W).astype(np.float64).sum(0)
+    bound_rows = 2.0 ** -11 * np.abs(c).sum(1) * 1.05 + 1e-3
+    assert (np.abs(c.sum(1) - want_rows) <= bound_rows).all()
+
+
+def test_fused_attention_at_full_size_agrees_with_the_four_kernel_chain(ttmi):
+    d = H // HEADS
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q, k, v = (torch.randn((B, HEADS, S, d), generator=g, device="cuda").half() for _ in range(3))
+    lens = np.random.default_rng(3).integers(1, S + 1, B)
+    mask = dev((-10000.0 * (np.arange(S)[None, :] >= lens[:, None])).astype(np.float32).reshape(B, 1, 1, S))
+    fused = torch.empty((B, S, H), dtype=torch.float16, device="cuda")
+    ok(ttmi.ttmi_fused_attention(ptr(q), ptr(k), ptr(v), ptr(mask), ptr(fused), None, B, HEADS, S, d, 0, 0.125,
+                                 TTMI_DTYPES["f16"], stream()))
+    score = torch.empty((B, HEADS, S, S), dtype=torch.float16, device="cuda")
+    ok(ttmi.ttmi_gemm_strided_batched(ptr(q), ptr(k), ptr(score), S, S, d, d, d, S, S * d, S * d, S * S, B * HEADS, 1, 0.125, 0.0,
+                                      TTMI_DTYPES["f16"], stream()))
+    ok(ttmi.ttmi_apply_mask_and_softmax(ptr(score), ptr(mask), B, HEADS, S, S, 1, 1.0, TTMI_DTYPES["f16"], stream()))
+    chain = torch.empty((B, S, H), dtype=torch.float16, device="cuda")
+    ok(ttmi.ttmi_gemm_batched_heads(ptr(score), ptr(v), ptr(chain), S, d, S, S, d, H, HEADS, HEADS * S * S, S * S, HEADS * S * d,
+                                    S * d, S * H, d, B, 0, 1.0, 0.0, TTMI_DTYPES["f16"], stream()))
+    # the chain rounds the scaled scores to fp16 before the softmax, the one-kernel form does not
+    assert max_abs(host(fused), host(chain)) < 8e-3
+    # rows of the softmax sum to one: with V = 1 every output is 1 (to the fp16 rounding of P)
+    ones = torch.ones_like(v)
+    ok(ttmi.ttmi_fused_attention(ptr(q), ptr(k), ptr(ones), ptr(mask), ptr(fused), None, B, HEADS, S, d, 0, 0.125,
+                                 TTMI_DTYPES["f16"], stream()))
+    assert max_abs(host(fused), 1.0) < 2e-3
+
+
+def test_layer_norm_rows_are_standardised_at_full_size(ttmi):
+    M = B * S
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = (torch.randn((M, H), generator=g, device="cuda") * 3 + 1).half()
+    res = torch.randn((M, H), generator=g, device="cuda").half()
+    bias = torch.randn(H, generator=g, device="cuda").half()
+    gamma, beta = torch.ones(H, dtype=torch.float16, device="cuda"), torch.zeros(H, dtype=torch.float16, device="cuda")
+    ok(ttmi.ttmi_add_bias_layer_norm(ptr(x), ptr(res), ptr(bias), ptr(gamma), ptr(beta), M, H, 1e-12, TTMI_DTYPES["f16"], stream()))
+    y = x.float()
+    torch.cuda.synchronize()
+    assert float(y.mean(1).abs().max()) < 1e-3
+    assert float((y.var(1, unbiased=False) - 1).abs().max()) < 2e-3

@@ -35,7 +35,7 @@ class QuantizedLinear {
   void Prepare() const;
   core::Tensor weight_, bias_;
   int act_ = -1;  // ttmi_act; -1 = none
-  mutable core::Tensor q_weight_, w_scales_, q_input_, acc_, act_scale_;
+  mutable core::Tensor q_weight_, w_scales_, q_input_, act_scale_;
   mutable bool prepared_ = false;
 };
 

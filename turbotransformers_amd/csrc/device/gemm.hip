@@ -787,6 +787,14 @@ constexpr int fast_lds_bytes() {
   return stage + (fast_epilogue_bytes<BM, BN, WM, WN>() > stage ? fast_epilogue_bytes<BM, BN, WM, WN>() : stage);
 }
 
+// Barrier that publishes DMA-filled LDS: every wavefront first waits for its own global->LDS loads
+// (vmcnt counts them; nothing obliges the compiler to place that wait in front of the barrier), then the
+// workgroup synchronises, so that afterwards any wavefront may read rows fetched by any other.
+__device__ __forceinline__ void dma_landed_barrier() {
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+  __syncthreads();
+}
+
 template <typename T, int BM, int BN, int WM, int WN, typename Epi>
 __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmArgs g, const Epi epi) {
   constexpr int NW = WM * WN, NT = NW * kWave;
@@ -804,9 +812,8 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   // Persistent workgroups: the grid holds at most as many workgroups as stay resident and each
   // walks over several tiles.  XCD x owns the contiguous tile range [x*per_xcd, (x+1)*per_xcd);
   // its workgroups (ids equal to x mod 8) stride through it together.  Between two tiles the
-  // first K step of the next tile is fetched (DMA into stage 0) while the epilogue of the
-  // finished tile runs out of the other half of LDS, and the epilogue's global stores drain
-  // under the next tile's K loop.
+  // first K step of the next tile is fetched (DMA into stage 0) before the epilogue of the
+  // finished tile runs out of the other half of LDS.
   const int tiles = g.tiles_m * g.tiles_n;
   // With fewer than kXcdRemapMinTiles tiles per problem the grid is simply one workgroup per tile.
   const bool remap = tiles >= kXcdRemapMinTiles;
@@ -931,7 +938,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-    __syncthreads();  // step 0 has landed; the previous tile's staging area has been read out
+    dma_landed_barrier();  // step 0 has landed; the previous tile's staging area has been read out
     if (ksteps > 1) issue(1);
     Chunk fa[2][TM], fb[2][TN];
     read_frags(smem, 0, fa[0], fb[0]);
@@ -948,7 +955,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
       read_frags(st, 3, fa[1], fb[1]);
       mma_step(fa[0], fb[0]);
       interleave();
-      __syncthreads();
+      dma_landed_barrier();  // the other stage is complete, and everyone has read all of this one
       if (kt + 2 < ksteps) issue(cur);
       read_frags(st_next, 0, fa[0], fb[0]);  // harmless on the last step
       mma_step(fa[1], fb[1]);
@@ -957,9 +964,13 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
     __syncthreads();  // all LDS reads of this tile are done
 
     const int next = logical + stride;
-    if (next < xcd_end) {  // stage 0 is free: fetch the next tile's first K step under the epilogue
+    if (next < xcd_end) {  // stage 0 is free: fetch the next tile's first K step
       point_at(next);
       issue(0);
+      // Let it land before the epilogue starts.  With an LDS DMA in flight the compiler puts a vmcnt(0) in
+      // front of every staging read of the epilogue, which would also wait for the previous strip's global
+      // stores, one round trip per strip; after this wait the strips' stores are issued back to back.
+      __builtin_amdgcn_s_waitcnt(0x0F70);
     }
     store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN>() - STAGE>(acc, bj, smem + STAGE, epi, g, z_epi, m0 + wm0,
                                                                          n0 + wn0, lane, wave);

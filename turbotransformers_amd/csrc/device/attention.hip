@@ -247,7 +247,12 @@ __global__ __launch_bounds__(256, 4) void fused_attention_kernel(const T* __rest
       float mx = st[0];
 #pragma unroll
       for (int e = 1; e < 16; ++e) mx = fmaxf(mx, st[e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      {
+        // the other half-wavefront holds the remaining 16 keys of this query: exchange through
+        // v_permlane32_swap (two VALU instructions) instead of an LDS permute and its wait
+        const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, mx), __builtin_bit_cast(unsigned, mx), false, false);
+        mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+      }
       // Lazy running maximum: the reference point m_run only moves when some query of the
       // wavefront would otherwise see exp2 arguments above kSlack (fp16: probabilities up to 2^kSlack are
       // as precise as smaller ones and the final division by the row sum cancels the choice of

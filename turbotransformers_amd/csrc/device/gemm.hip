@@ -23,6 +23,8 @@
 // cover neighbouring tiles and share A rows / the weight matrix in that XCD's L2.
 #include <map>
 #include <mutex>
+#include <set>
+#include <utility>
 
 #include "common.h"
 
@@ -980,6 +982,19 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
 }
 
 // ------------------------------------------------------------------------ launching -----
+// Kernels that use more than 64 KB of dynamic LDS need the limit raised once per kernel and device.
+static int allow_large_lds(const void* kern, int bytes) {
+  static std::mutex mu;
+  static std::set<std::pair<const void*, int>> done;
+  int dev = 0;
+  TTMI_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count({kern, dev}) != 0) return 0;
+  TTMI_HIP(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  done.insert({kern, dev});
+  return 0;
+}
+
 template <typename T, int BM, int BN, int WM, int WN, bool B_KN, bool ALIGNED, typename Epi>
 static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   constexpr int NT = WM * WN * kWave;
@@ -992,11 +1007,8 @@ static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   constexpr int DEPTH = (BM * BN <= 64 * 64 && ALIGNED) ? 2 : 1;
   auto kern = gemm_kernel<T, BM, BN, WM, WN, B_KN, ALIGNED, DEPTH, Epi>;
   if (LDS > 64 * 1024) {
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-      TTMI_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-      attr_set = true;
-    }
+    const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
+    if (rc != 0) return rc;
   }
   hipLaunchKernelGGL(kern, dim3(grid_x, 1, (unsigned)batch), dim3(NT), LDS, s, g, epi);
   return launch_status("gemm_kernel");
@@ -1031,11 +1043,8 @@ static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
           : (unsigned)tiles;
   auto kern = gemm_fast_kernel<T, BM, BN, WM, WN, Epi>;
   if (LDS > 64 * 1024) {
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-      TTMI_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-      attr_set = true;
-    }
+    const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
+    if (rc != 0) return rc;
   }
   hipLaunchKernelGGL(kern, dim3(grid_x, 1, (unsigned)batch), dim3(NT), LDS, s, g, epi);
   return launch_status("gemm_fast_kernel");
@@ -1112,10 +1121,9 @@ static int launch_fast_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hi
   EpiPartial part{ws, (int64_t)g.m * g.n, g.n, vec};
   constexpr int LDS = fast_lds_bytes<128, 128, 2, 2>();
   auto kern = gemm_fast_kernel<T, 128, 128, 2, 2, EpiPartial>;
-  static bool attr_set = false;  // per instantiation
-  if (!attr_set) {
-    TTMI_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-    attr_set = true;
+  {
+    const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
+    if (rc != 0) return rc;
   }
   // one workgroup per (tile, slice): the persistent loop runs once
   const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;

@@ -327,6 +327,13 @@ TTMI_API int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t 
 TTMI_API int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev,
                                   const float* w_scale, const float* bias, int act, int64_t m, int64_t n, int64_t k,
                                   int64_t lda, int64_t ldb, int64_t ldc, void* stream);
+/* ttmi_gemm_i8_dequant_qkv_split: the QKV projection of the quantized attention: the dequantised product plus
+ *   bias[3*heads*head_dim] written straight to q,k,v[B,heads,seq,head_dim] (fp32), i.e. ttmi_gemm_i8_dequant
+ *   without bias followed by ttmi_split_add_bias_transpose_for_score, with the same bits. */
+TTMI_API int ttmi_gemm_i8_dequant_qkv_split(const int8_t* a, const int8_t* b, const float* act_scale_dev,
+                                            const float* w_scale, const float* bias, float* q, float* k_out,
+                                            float* v, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                                            int64_t seq, int64_t heads, int64_t head_dim, void* stream);
 TTMI_API int ttmi_dequant_bias(const int32_t* acc, const float* act_scale_dev, const float* w_scale,
                                const float* bias, float* out, int64_t m, int64_t n, void* stream);
 

@@ -376,6 +376,35 @@ def test_gemm_i8_dequant_equals_unfused(ttmi, oracle, M, N, K, with_bias):
         assert max_abs(host(fused), oracle.add_bias_act(want, np.zeros(N, np.float32), 0)) <= 2e-5 * max(1.0, float(np.abs(want).max()))
 
 
+@pytest.mark.parametrize("B,S,h,d", [(20, 128, 12, 64), (3, 17, 2, 8), (2, 9, 3, 20)])
+def test_gemm_i8_dequant_qkv_split_equals_the_two_kernels(ttmi, oracle, B, S, h, d):
+    """int8 QKV projection with dequantisation, bias and head split in its store: the bits of
+    ttmi_gemm_i8_dequant (no bias) followed by ttmi_split_add_bias_transpose_for_score, and the oracle's values."""
+    rng = np.random.default_rng(B + S)
+    H = h * d
+    M, N, K = B * S, 3 * H, H if H % 16 == 0 else 48
+    a = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    b = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    sx = np.array([0.0123, 0.0], np.float32)
+    sw = (rng.random(N, np.float32) + 0.5) * 1e-3
+    bias = rng.standard_normal(N).astype(np.float32)
+    dA, dB, dsx, dsw, dbias = dev(a), dev(b), dev(sx), dev(sw), dev(bias)
+    flat = torch.empty((M, N), device="cuda")
+    ok(ttmi.ttmi_gemm_i8_dequant(ptr(dA), ptr(dB), ptr(flat), ptr(dsx), ptr(dsw), None, -1, M, N, K, K, K, N, stream()))
+    two = [torch.empty((B, h, S, d), device="cuda") for _ in range(3)]
+    ok(ttmi.ttmi_split_add_bias_transpose_for_score(ptr(flat), ptr(dbias), ptr(two[0]), ptr(two[1]), ptr(two[2]), B, S, h, d,
+                                                    TTMI_DTYPES["f32"], stream()))
+    one = [torch.full((B, h, S, d), 7.0, device="cuda") for _ in range(3)]
+    ok(ttmi.ttmi_gemm_i8_dequant_qkv_split(ptr(dA), ptr(dB), ptr(dsx), ptr(dsw), ptr(dbias), ptr(one[0]), ptr(one[1]), ptr(one[2]),
+                                           M, N, K, K, K, S, h, d, stream()))
+    for x, y in zip(one, two):
+        assert torch.equal(x, y)
+    want = oracle.split_add_bias_transpose(oracle.dequant_bias(oracle.gemm_i8(a, b), sx[0], sw, np.zeros(N, np.float32)), bias,
+                                           B, S, h, d)
+    for x, y in zip(one, want):
+        assert max_abs(host(x), y) <= 1e-5 * max(1.0, float(np.abs(y).max()))
+
+
 def test_int8_linear_pipeline(ttmi, oracle):
     """quantize -> int8 GEMM -> dequant+bias, against the oracle's statement of the same scheme."""
     rng = np.random.default_rng(3)

@@ -380,6 +380,28 @@ struct EpiDequant {
   }
 };
 
+// The same dequantisation feeding the head split: q,k,v[B,h,S,d] (fp32) = split(float(acc) * act_scale *
+// w_scale[n] + bias[n]), the QKV projection of the quantized attention without the [T,3H] round trip.
+// Scaling first, bias second -- the order of dequant_bias followed by SplitAddBiasTransposeForScore.
+struct EpiDequantQkvSplit {
+  using Acc = int;
+  EpiQkvSplit<float, false> split;  // its bias is added here, after the scaling
+  const float* act_scale;           // device scalar
+  const float* w_scale;             // [N]
+  __device__ __forceinline__ const float* bias_ptr() const { return nullptr; }
+  __device__ __forceinline__ void store8(int z, int m, int n, int (&v)[8], int valid) const {
+#pragma clang fp contract(off)  // the bias is added to the ROUNDED product, as the separate kernel does
+    const float sx = act_scale[0];
+    float r[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float scaled = (float)v[j] * sx * w_scale[j < valid ? n + j : n];
+      r[j] = scaled + split.bias[j < valid ? n + j : n];
+    }
+    split.store8(z, m, n, r, valid);
+  }
+};
+
 // -------------------------------------------------------------------------- kernel ------
 // LDS rows are 128 bytes and the LDS has 64 four-byte banks (256 bytes per bank cycle): rows r and
 // r+2 start on the same bank.  A 128-bit operand read is served 16 lanes (= 16 consecutive tile
@@ -1470,6 +1492,29 @@ int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float
   g.lda = lda; g.ldb = ldb;
   g.inner = 1;
   EpiDequant epi{c, act_scale_dev, w_scale, bias, ldc, aligned16(c) && ldc % 4 == 0, act};
+  const bool aligned = aligned16(a) && aligned16(b) && lda % 16 == 0 && ldb % 16 == 0 && k % 16 == 0;
+  return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
+}
+
+int ttmi_gemm_i8_dequant_qkv_split(const int8_t* a, const int8_t* b, const float* act_scale_dev, const float* w_scale,
+                                   const float* bias, float* q, float* k_out, float* v, int64_t m, int64_t n, int64_t k,
+                                   int64_t lda, int64_t ldb, int64_t seq, int64_t heads, int64_t head_dim, void* stream) {
+  TTMI_REQUIRE(a && b && act_scale_dev && w_scale && bias && q && k_out && v, "null tensor");
+  TTMI_REQUIRE(m < (1ll << 31) && n < (1ll << 31) && k < (1ll << 31), "dimension too large");
+  TTMI_REQUIRE(lda >= k && ldb >= k, "leading dimension too small");
+  TTMI_REQUIRE(seq > 0 && heads > 0 && head_dim > 0 && n == 3 * heads * head_dim, "N must be 3*heads*head_dim");
+  TTMI_REQUIRE(m % seq == 0, "M must be a multiple of seq");
+  GemmArgs g{};
+  g.a = (const char*)a;
+  g.b = (const char*)b;
+  g.m = (int)m; g.n = (int)n; g.k = (int)k;
+  g.lda = lda; g.ldb = ldb;
+  g.inner = 1;
+  const int hidden = (int)(heads * head_dim);
+  const bool vec = aligned16(q) && aligned16(k_out) && aligned16(v) && head_dim % 8 == 0;
+  EpiDequantQkvSplit epi{{q, k_out, v, bias, nullptr, (int)seq, (int)heads, (int)head_dim, hidden, FastDiv((uint32_t)seq),
+                          FastDiv((uint32_t)hidden), FastDiv((uint32_t)head_dim), vec, 0},
+                         act_scale_dev, w_scale};
   const bool aligned = aligned16(a) && aligned16(b) && lda % 16 == 0 && ldb % 16 == 0 && k % 16 == 0;
   return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
 }

@@ -40,24 +40,39 @@ void QuantizedLinear::Prepare() const {
   prepared_ = true;
 }
 
-void QuantizedLinear::operator()(const Tensor& input_tensor, Tensor* output_tensor) const {
+const int8_t* QuantizedLinear::QuantizeInput(const Tensor& input_tensor) const {
   kernels::RequireGpu(input_tensor, "QuantizedLinear");
   Prepare();
-  const int64_t k = weight_.shape(0), n = weight_.shape(1);
+  const int64_t k = weight_.shape(0);
   TT_ENFORCE_EQ(input_tensor.shape(-1), k, "input width and weight rows differ");
   const int64_t m = input_tensor.numel() / k;
-  const DLDeviceType dev = input_tensor.device_type();
-  const int id = input_tensor.device_id();
-  int8_t* qx = q_input_.Reshape<int8_t>({m, k}, dev, id, "QuantizedLinear/q_input");
+  int8_t* qx = q_input_.Reshape<int8_t>({m, k}, input_tensor.device_type(), input_tensor.device_id(), "QuantizedLinear/q_input");
+  TT_DEVICE_CALL(ttmi_quantize_rows_i8(input_tensor.data<float>(), qx, act_scale_.mutableData<float>(), m, k, Stream()));
+  return qx;
+}
+
+void QuantizedLinear::operator()(const Tensor& input_tensor, Tensor* output_tensor) const {
+  const int8_t* qx = QuantizeInput(input_tensor);
+  const int64_t k = weight_.shape(0), n = weight_.shape(1), m = input_tensor.numel() / k;
   std::vector<int64_t> shape;
   for (size_t i = 0; i + 1 < input_tensor.n_dim(); ++i) shape.push_back(input_tensor.shape((int)i));
   shape.push_back(n);
-  float* out = output_tensor->Reshape<float>(shape, dev, id, "QuantizedLinear/Reshape");
-  float* scale = act_scale_.mutableData<float>();
-  TT_DEVICE_CALL(ttmi_quantize_rows_i8(input_tensor.data<float>(), qx, scale, m, k, Stream()));
+  float* out = output_tensor->Reshape<float>(shape, input_tensor.device_type(), input_tensor.device_id(), "QuantizedLinear/Reshape");
   // int8 GEMM with the dequantisation folded into its store: the int32 accumulators stay on chip
-  TT_DEVICE_CALL(ttmi_gemm_i8_dequant(qx, q_weight_.data<int8_t>(), out, scale, w_scales_.data<float>(),
+  TT_DEVICE_CALL(ttmi_gemm_i8_dequant(qx, q_weight_.data<int8_t>(), out, act_scale_.data<float>(), w_scales_.data<float>(),
                                       bias_.is_null() ? nullptr : bias_.data<float>(), act_, m, n, k, k, k, n, Stream()));
+}
+
+void QuantizedLinear::ProjectToHeads(const Tensor& input_tensor, const Tensor& bias, int64_t seq, int64_t heads, Tensor* q,
+                                     Tensor* k_out, Tensor* v) const {
+  TT_ENFORCE(bias_.is_null() && act_ < 0, "ProjectToHeads takes the bias as an argument");
+  const int8_t* qx = QuantizeInput(input_tensor);
+  const int64_t k = weight_.shape(0), n = weight_.shape(1), m = input_tensor.numel() / k;
+  TT_ENFORCE_EQ(bias.numel(), n, "bias and weight shape mismatch");
+  TT_ENFORCE(n % (3 * heads) == 0 && q->numel() == m * (n / 3), "q,k,v must be shaped [B, heads, S, d]");
+  TT_DEVICE_CALL(ttmi_gemm_i8_dequant_qkv_split(qx, q_weight_.data<int8_t>(), act_scale_.data<float>(), w_scales_.data<float>(),
+                                                bias.data<float>(), q->mutableData<float>(), k_out->mutableData<float>(),
+                                                v->mutableData<float>(), m, n, k, k, k, seq, heads, n / (3 * heads), Stream()));
 }
 
 void QuantizedBertAttention::operator()(const Tensor& input_tensor, const Tensor& attention_mask, Tensor* output,
@@ -68,13 +83,11 @@ void QuantizedBertAttention::operator()(const Tensor& input_tensor, const Tensor
   const int64_t B = input_tensor.shape(0), S = input_tensor.shape(1), H = input_tensor.shape(2), d = H / heads_;
   const DLDeviceType dev = input_tensor.device_type();
   const int id = input_tensor.device_id();
-  // QKV projection (int8) -> fp32 [B,S,3,H]; then the reference's unfused fp32 chain
-  qkv_(input_tensor, &qkv_out_);
-  qkv_out_.Reshape<float>({B, S, 3, H}, dev, id, "self/qkv_out1/Reshape");
+  // QKV projection (int8) with bias and head split in its store; then the reference's unfused fp32 chain
   q_.Reshape<float>({B, heads_, S, d}, dev, id, "self/q/Reshape");
   k_.Reshape<float>({B, heads_, S, d}, dev, id, "self/k/Reshape");
   v_.Reshape<float>({B, heads_, S, d}, dev, id, "self/v/Reshape");
-  kernels::SplitAddBiasTransposeForScore(qkv_out_, qkv_bias_, q_, k_, v_);
+  qkv_.ProjectToHeads(input_tensor, qkv_bias_, S, heads_, &q_, &k_, &v_);
   Tensor* score = attn != nullptr ? attn : &score_scratch_;
   score->Reshape<float>({B, heads_, S, S}, dev, id, "batch_gemm3/Reshape");
   kernels::BatchMatMul(q_, false, k_, true, 1.0f / std::sqrt((float)d), score, 0.f);

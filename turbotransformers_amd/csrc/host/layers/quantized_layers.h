@@ -28,11 +28,16 @@ class QuantizedLinear {
   QuantizedLinear(core::Tensor weight, core::Tensor bias, const std::string& activation);
   // output[tokens, out] (fp32) = act(dequant(q(input) * q(weight)^T) + bias)
   void operator()(const core::Tensor& input_tensor, core::Tensor* output_tensor) const;
+  // A [hidden, 3*hidden] projection written as q,k,v[B, heads, S, d] = split(dequant(...) + bias): the Linear and
+  // SplitAddBiasTransposeForScore of the attention in one kernel.  q,k,v are already shaped.
+  void ProjectToHeads(const core::Tensor& input_tensor, const core::Tensor& bias, int64_t seq, int64_t heads, core::Tensor* q,
+                      core::Tensor* k, core::Tensor* v) const;
   int64_t in_features() const { return weight_.shape(0); }
   int64_t out_features() const { return weight_.shape(1); }
 
  private:
   void Prepare() const;
+  const int8_t* QuantizeInput(const core::Tensor& input_tensor) const;  // -> q_input_, scale in act_scale_
   core::Tensor weight_, bias_;
   int act_ = -1;  // ttmi_act; -1 = none
   mutable core::Tensor q_weight_, w_scales_, q_input_, act_scale_;
@@ -54,7 +59,7 @@ class QuantizedBertAttention {
   QuantizedLinear qkv_, dense_;
   core::Tensor qkv_bias_, dense_bias_, ln_weight_, ln_bias_;
   int64_t heads_;
-  mutable core::Tensor qkv_out_, q_, k_, v_, ctx_, merged_, score_scratch_;
+  mutable core::Tensor q_, k_, v_, ctx_, merged_, score_scratch_;
   mutable std::mutex mutex_;
 };
 

@@ -130,6 +130,45 @@ def test_npz_reader_matches_numpy(tmp_path):
     assert set(loaded) == set(arrays)
     for k, v in arrays.items():
         assert loaded[k].dtype == v.dtype and np.array_equal(loaded[k], v)
+    # deflated members: what numpy.savez_compressed and the reference's converter
+    # (tools/convert_huggingface_bert_pytorch_to_npz.py:71) write; a larger, compressible array as well
+    arrays["big"] = np.tile(rng.standard_normal(1000).astype(np.float32), 300).reshape(600, 500)
     np.savez_compressed(path, **arrays)
-    with pytest.raises(RuntimeError, match="compressed"):
-        cxx.load_npz(path)
+    loaded = cxx.load_npz(path)
+    assert set(loaded) == set(arrays)
+    for k, v in arrays.items():
+        assert loaded[k].dtype == v.dtype and np.array_equal(loaded[k], v)
+    # a truncated archive is an error, not a crash
+    data = open(path, "rb").read()
+    bad = str(tmp_path / "bad.npz")
+    open(bad, "wb").write(data[:len(data) // 2])
+    with pytest.raises(RuntimeError):
+        cxx.load_npz(bad)
+
+
+def test_converter_writes_the_reference_key_scheme(tmp_path):
+    """tools/convert_huggingface_bert_pytorch_to_npz.py:44-71: q/k/v packed into qkv.weight [hidden, 3*hidden] and
+    qkv.bias, other dense weights transposed to [in, out]; the (deflated) file reads back through the C++ loader."""
+    import torch
+    from transformers import BertConfig, BertModel
+    import turbo_transformers.turbo_transformers_cxx as cxx
+    from turbotransformers_amd.convert_huggingface_bert_to_npz import save_bert_npz
+    torch.manual_seed(0)
+    model = BertModel(BertConfig(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, intermediate_size=128, vocab_size=100))
+    path = str(tmp_path / "m.npz")
+    save_bert_npz(model, path)
+    got = cxx.load_npz(path)
+    sd = {k: v.detach().numpy() for k, v in model.named_parameters()}
+    assert not any(".attention.self." in k for k in got)
+    for i in range(2):
+        p = "encoder.layer.%d." % i
+        want = np.concatenate([sd[p + "attention.self.%s.weight" % x] for x in ("query", "key", "value")], 0).T
+        assert np.array_equal(got[p + "attention.qkv.weight"], want) and want.shape == (64, 192)
+        assert np.array_equal(got[p + "attention.qkv.bias"],
+                              np.concatenate([sd[p + "attention.self.%s.bias" % x] for x in ("query", "key", "value")]))
+        assert np.array_equal(got[p + "intermediate.dense.weight"], sd[p + "intermediate.dense.weight"].T)
+        assert np.array_equal(got[p + "output.dense.weight"], sd[p + "output.dense.weight"].T)
+        assert np.array_equal(got[p + "attention.output.dense.weight"], sd[p + "attention.output.dense.weight"].T)
+    assert np.array_equal(got["pooler.dense.weight"], sd["pooler.dense.weight"].T)
+    assert np.array_equal(got["embeddings.word_embeddings.weight"], sd["embeddings.word_embeddings.weight"])
+

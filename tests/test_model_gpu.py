@@ -268,31 +268,13 @@ def test_albert_model_vs_huggingface(tt, dtype):
     assert max_abs(host(pooled), host(want.pooler_output)) < tol
 
 
-def _npz_weights(model):
-    """HuggingFace BertModel -> the npz key scheme of tools/convert_huggingface_bert_pytorch_to_npz.py:44-71."""
-    sd = {k: v.detach().float().cpu().numpy() for k, v in model.named_parameters()}
-    out = {}
-    for k, v in sd.items():
-        if ".attention.self." in k:
-            continue
-        if k.endswith("dense.weight"):
-            v = np.ascontiguousarray(v.T)
-        out[k] = v
-    n = model.config.num_hidden_layers
-    for i in range(n):
-        p = f"encoder.layer.{i}.attention."
-        out[p + "qkv.weight"] = np.ascontiguousarray(np.concatenate(
-            [sd[p + f"self.{x}.weight"] for x in ("query", "key", "value")], 0).T)
-        out[p + "qkv.bias"] = np.concatenate([sd[p + f"self.{x}.bias"] for x in ("query", "key", "value")])
-    return out
-
-
 def test_cxx_bert_model_api_from_npz(tt, tmp_path):
     """The C++ BertModel(file, device, n_layers, n_heads) of example/cpp: ragged ids in, pooled or
     full hidden vector out; also from_npz on the Python side."""
     model, cfg = _hf_bert(2, seed=12, hidden_size=128, num_attention_heads=4, intermediate_size=512, vocab_size=300)
+    from turbotransformers_amd.convert_huggingface_bert_to_npz import save_bert_npz
     path = str(tmp_path / "bert.npz")
-    np.savez(path, **_npz_weights(model))
+    save_bert_npz(model, path)  # deflated members, like the reference's converter writes
     cxx_model = tt.cxx.CxxBertModel(path, cfg.num_hidden_layers, cfg.num_attention_heads)
     ids = [[12, 101, 7, 55, 2, 9], [5, 6, 250]]
     vec = np.array(cxx_model(ids, [], [], "First", True))

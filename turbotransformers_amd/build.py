@@ -108,7 +108,7 @@ def build_host(jobs=8, verbose=True):
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(compile_one, sources))
     _run([CXX, "-shared", "-o", host_module_path()] + objs +
-         ["-L", LIB_DIR, "-lttmi", "-Wl,-rpath,$ORIGIN/lib", "-lpthread"])
+         ["-L", LIB_DIR, "-lttmi", "-Wl,-rpath,$ORIGIN/lib", "-lpthread", "-lz"])
     if verbose:
         print("built", host_module_path())
     return host_module_path()

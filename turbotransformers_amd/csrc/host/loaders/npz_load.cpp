@@ -1,7 +1,11 @@
 #include "loaders/npz_load.h"
 
+#include <zlib.h>
+
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 #include "core/enforce.h"
 
@@ -22,6 +26,43 @@ struct File {
   int64_t Tell() { return ftello(f); }
   void Read(void* dst, size_t n) { TT_ENFORCE_EQ(std::fread(dst, 1, n, f), n, "unexpected end of file"); }
 };
+
+// A member that has been inflated into memory, read like a file.
+struct MemReader {
+  const unsigned char* p;
+  size_t left;
+  void Read(void* dst, size_t n) {
+    TT_ENFORCE(n <= left, "unexpected end of a compressed member");
+    std::memcpy(dst, p, n);
+    p += n;
+    left -= n;
+  }
+};
+
+// Raw deflate stream (ZIP method 8) -> `usize` bytes.
+std::vector<unsigned char> Inflate(const std::vector<unsigned char>& in, uint64_t usize) {
+  std::vector<unsigned char> out(usize);
+  z_stream zs;
+  std::memset(&zs, 0, sizeof(zs));
+  TT_ENFORCE_EQ(inflateInit2(&zs, -MAX_WBITS), Z_OK, "inflateInit2 failed");
+  size_t in_pos = 0, out_pos = 0;
+  int rc = Z_OK;
+  while (rc != Z_STREAM_END) {  // avail_in / avail_out are 32-bit: feed members larger than 4 GiB in pieces
+    const size_t in_chunk = std::min<size_t>(in.size() - in_pos, 1u << 30), out_chunk = std::min<size_t>(out.size() - out_pos, 1u << 30);
+    zs.next_in = const_cast<unsigned char*>(in.data()) + in_pos;
+    zs.avail_in = (uInt)in_chunk;
+    zs.next_out = out.data() + out_pos;
+    zs.avail_out = (uInt)out_chunk;
+    rc = inflate(&zs, Z_NO_FLUSH);
+    in_pos += in_chunk - zs.avail_in;
+    out_pos += out_chunk - zs.avail_out;
+    if (rc != Z_OK && rc != Z_STREAM_END) break;
+    if (rc == Z_OK && in_chunk - zs.avail_in == 0 && out_chunk - zs.avail_out == 0) break;  // no progress: truncated
+  }
+  inflateEnd(&zs);
+  TT_ENFORCE(rc == Z_STREAM_END && out_pos == usize, "corrupt compressed member (zlib status %d)", rc);
+  return out;
+}
 
 template <typename T>
 T Get(const unsigned char* p) {
@@ -46,7 +87,8 @@ void ApplyZip64(const unsigned char* extra, size_t extra_len, uint64_t* usize, u
   }
 }
 
-NpyArray ParseNpy(File& file, uint64_t size) {
+template <typename Reader>
+NpyArray ParseNpy(Reader& file, uint64_t size) {
   unsigned char head[12];
   file.Read(head, 10);
   TT_ENFORCE(std::memcmp(head, "\x93NUMPY", 6) == 0, "not an npy member");
@@ -145,8 +187,10 @@ std::map<std::string, NpyArray> LoadNpz(const std::string& filename) {
     if (extra_len) file.Read(extra.data(), extra_len);
     ApplyZip64(extra.data(), extra_len, &usize, &csize, &local);
     pos += 46 + name_len + extra_len + comment_len;
-    TT_ENFORCE_EQ(method, 0, "%s: member %s is compressed; save with numpy.savez (not savez_compressed)", filename.c_str(),
-                  name.c_str());
+    // numpy.savez stores members (method 0); numpy.savez_compressed, which the reference's converter
+    // uses (tools/convert_huggingface_bert_pytorch_to_npz.py:71), deflates them (method 8)
+    TT_ENFORCE(method == 0 || method == 8, "%s: member %s uses zip compression method %d (stored and deflate are read)",
+               filename.c_str(), name.c_str(), (int)method);
     // Local header: 30 bytes + its own name/extra lengths, then the data.
     unsigned char lh[30];
     file.Seek((int64_t)local);
@@ -154,7 +198,15 @@ std::map<std::string, NpyArray> LoadNpz(const std::string& filename) {
     TT_ENFORCE_EQ(Get<uint32_t>(lh), 0x04034b50u, "bad local file header");
     file.Seek((int64_t)local + 30 + Get<uint16_t>(lh + 26) + Get<uint16_t>(lh + 28));
     if (name.size() > 4 && name.compare(name.size() - 4, 4, ".npy") == 0) name.resize(name.size() - 4);
-    out.emplace(name, ParseNpy(file, usize));
+    if (method == 0) {
+      out.emplace(name, ParseNpy(file, usize));
+    } else {
+      std::vector<unsigned char> packed(csize);
+      if (csize) file.Read(packed.data(), csize);
+      const std::vector<unsigned char> raw = Inflate(packed, usize);
+      MemReader mem{raw.data(), raw.size()};
+      out.emplace(name, ParseNpy(mem, usize));
+    }
   }
   return out;
 }

@@ -1,8 +1,8 @@
 // Reader for .npz weight files (the on-disk format of the reference's C++ model and of
 // from_npz; the reference reads them with the cnpy library, loaders/npz_load.h:23-75).
-// An .npz is a ZIP archive of .npy members; numpy.savez stores them uncompressed (method 0,
-// ZIP64 sizes), which is the only form read here.  Supports little-endian float32, float16
-// and int64 arrays in C order.
+// An .npz is a ZIP archive of .npy members: stored (numpy.savez) or deflated (numpy.savez_compressed,
+// what the reference's converter writes), with ZIP64 sizes where needed.  Supports little-endian float32,
+// float16 and int64 arrays in C order.
 #pragma once
 
 #include <cstdint>
@@ -26,7 +26,7 @@ struct NpyArray {
 };
 
 // name (without the ".npy" suffix) -> array.  Throws core::EnforceNotMet on malformed input,
-// compressed members or unsupported dtypes.
+// other compression methods or unsupported dtypes.
 std::map<std::string, NpyArray> LoadNpz(const std::string& filename);
 
 }  // namespace loaders

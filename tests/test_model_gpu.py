@@ -294,6 +294,34 @@ def test_cxx_bert_model_api_from_npz(tt, tmp_path):
     assert max_abs(host(seq)[0], host(want.last_hidden_state)[0]) < 1e-3
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.float16, 2e-2)])
+def test_roberta_model_vs_huggingface(tt, dtype, tol):
+    """python/tests/roberta_model_test.py: a random-init HuggingFace RobertaModel, converted, same ids and padding
+    mask.  Position ids follow RoBERTa's rule (pad tokens keep padding_idx, the others count up from it)."""
+    from transformers import RobertaConfig, RobertaModel
+    torch.manual_seed(31)
+    cfg = RobertaConfig(num_hidden_layers=2, hidden_size=128, num_attention_heads=4, intermediate_size=512, vocab_size=200,
+                        max_position_embeddings=80, hidden_act="gelu_pytorch_tanh", hidden_dropout_prob=0.0,
+                        attention_probs_dropout_prob=0.0, attn_implementation="eager")
+    model = RobertaModel(cfg).eval().cuda().to(dtype)
+    ref = RobertaModel(cfg).eval().cuda()
+    ref.load_state_dict({k: v.float() for k, v in model.state_dict().items()})
+    g = torch.Generator().manual_seed(32)
+    ids = torch.randint(2, cfg.vocab_size, (3, 40), generator=g)
+    ids[1, 25:] = cfg.pad_token_id
+    ids[2, 7:] = cfg.pad_token_id
+    ids = ids.cuda()
+    mask = ids.ne(cfg.pad_token_id).long()
+    with torch.no_grad():
+        want = ref(input_ids=ids, attention_mask=mask)
+    tmodel = tt.RobertaModel.from_torch(model, torch.device("cuda:0"))
+    seq, pooled = tmodel(ids, attention_mask=mask)[:2]
+    assert seq.dtype == dtype
+    valid = host(mask).astype(bool)
+    assert max_abs(host(seq)[valid], host(want.last_hidden_state)[valid]) < tol
+    assert max_abs(host(pooled), host(want.pooler_output)) < tol
+
+
 def test_out_of_range_id_is_reported(tt):
     model, cfg = _hf_bert(1, seed=2)
     tmodel = tt.BertModel.from_torch(model, torch.device("cuda:0"), "turbo")

@@ -322,6 +322,34 @@ def test_roberta_model_vs_huggingface(tt, dtype, tol):
     assert max_abs(host(pooled), host(want.pooler_output)) < tol
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.float16, 2e-2)])
+def test_distilbert_model_vs_huggingface(tt, dtype, tol):
+    """python/tests/distill_bert_model_test.py: a random-init HuggingFace DistilBertModel mapped onto the BERT
+    layers (no token types, other parameter names), same ids and padding mask."""
+    from transformers import DistilBertConfig, DistilBertModel
+    torch.manual_seed(41)
+    cfg = DistilBertConfig(n_layers=2, dim=128, n_heads=4, hidden_dim=512, vocab_size=200, max_position_embeddings=64,
+                           activation="gelu_pytorch_tanh", dropout=0.0, attention_dropout=0.0, attn_implementation="eager")
+    model = DistilBertModel(cfg).eval().cuda().to(dtype)
+    ref = DistilBertModel(cfg).eval().cuda()
+    ref.load_state_dict({k: v.float() for k, v in model.state_dict().items()})
+    ids = torch.randint(0, cfg.vocab_size, (3, 33), generator=torch.Generator().manual_seed(42)).cuda()
+    mask = torch.ones(3, 33, dtype=torch.int64)
+    mask[1, 20:] = 0
+    mask = mask.cuda()
+    with torch.no_grad():
+        want = ref(input_ids=ids, attention_mask=mask).last_hidden_state
+    tmodel = tt.DistilBertModel.from_torch(model, torch.device("cuda:0"))
+    seq = tmodel(ids, attention_masks=mask)[0]
+    assert seq.dtype == dtype
+    valid = host(mask).astype(bool)
+    assert max_abs(host(seq)[valid], host(want)[valid]) < tol
+    # no mask given = all ones
+    with torch.no_grad():
+        want = ref(input_ids=ids).last_hidden_state
+    assert max_abs(host(tmodel(ids)[0]), host(want)) < tol
+
+
 def test_out_of_range_id_is_reported(tt):
     model, cfg = _hf_bert(1, seed=2)
     tmodel = tt.BertModel.from_torch(model, torch.device("cuda:0"), "turbo")

@@ -7,6 +7,7 @@ from .modeling_albert import (AlbertEmbeddings, AlbertAttention, AlbertLayer, Al
 from .qmodeling_bert import QBertIntermediate, QBertOutput, QBertAttention, QBertLayer, QBertEncoder, QBertModel
 from .modules import MultiHeadedAttention, PositionwiseFeedForward, DistrillFFN
 from .modeling_roberta import RobertaModel
+from .modeling_distillbert import DistilBertModel
 from .return_type import ReturnType
 
 __all__ = [
@@ -14,5 +15,5 @@ __all__ = [
     'BertModelNoPooler', 'ReturnType', 'BertPooler', 'SequencePool', 'PoolingType', 'MultiHeadedAttentionSmartBatch',
     'BertLayerSmartBatch', 'BertEncoderSmartBatch', 'BertModelNoPoolerSmartBatch', 'BertModelSmartBatch',
     'QBertIntermediate', 'QBertOutput', 'QBertAttention', 'QBertLayer', 'QBertEncoder', 'QBertModel',
-    'MultiHeadedAttention', 'PositionwiseFeedForward', 'DistrillFFN', 'AlbertEmbeddings', 'AlbertAttention', 'AlbertLayer', 'AlbertLayerGroup', 'AlbertTransformer', 'AlbertModel', 'RobertaModel',
+    'MultiHeadedAttention', 'PositionwiseFeedForward', 'DistrillFFN', 'AlbertEmbeddings', 'AlbertAttention', 'AlbertLayer', 'AlbertLayerGroup', 'AlbertTransformer', 'AlbertModel', 'RobertaModel', 'DistilBertModel',
 ]

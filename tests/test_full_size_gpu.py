@@ -163,3 +163,37 @@ def test_layer_norm_rows_are_standardised_at_full_size(ttmi):
     torch.cuda.synchronize()
     assert float(y.mean(1).abs().max()) < 1e-3
     assert float((y.var(1, unbiased=False) - 1).abs().max()) < 2e-3
+
+
+def test_repeated_launches_give_the_same_bits(ttmi):
+    """A race between the DMA fills of LDS and their readers, or between the stores of one tile and the next
+    tile's loads, shows up as run-to-run differences: ten launches of the large GEMM shapes (with the epilogues the
+    encoder uses) and of the attention kernel must agree bit for bit."""
+    import ctypes
+    from turbotransformers_amd import capi
+    M = B * S
+    g = torch.Generator(device="cuda").manual_seed(11)
+    for N, K in [(3072, 768), (768, 3072), (2304, 768)]:
+        A = torch.randn((M, K), generator=g, device="cuda").half()
+        W = (torch.randn((N, K), generator=g, device="cuda") / K ** 0.5).half()
+        bias = torch.randn(N, generator=g, device="cuda").half()
+        args = capi.EpilogueArgs()
+        args.bias = bias.data_ptr()
+        args.act = capi.ACT_GELU
+        first = None
+        for _ in range(10):
+            C = torch.empty((M, N), dtype=torch.float16, device="cuda")
+            ok(ttmi.ttmi_gemm_fused(ptr(A), ptr(W), ptr(C), M, N, K, K, K, N, capi.EPI_BIAS_ACT, ctypes.byref(args),
+                                    TTMI_DTYPES["f16"], stream()))
+            first = C if first is None else first
+            assert torch.equal(C, first)
+    d = H // HEADS
+    q, k, v = (torch.randn((B, HEADS, S, d), generator=g, device="cuda").half() for _ in range(3))
+    first = None
+    for _ in range(5):
+        out = torch.empty((B, S, H), dtype=torch.float16, device="cuda")
+        ok(ttmi.ttmi_fused_attention(ptr(q), ptr(k), ptr(v), None, ptr(out), None, B, HEADS, S, d, 0, 0.125, TTMI_DTYPES["f16"],
+                                     stream()))
+        first = out if first is None else first
+        assert torch.equal(out, first)
+

@@ -121,11 +121,30 @@ TTMI_API int ttmi_add_bias_layer_norm_residual32(void* out, const float* residua
  * fill the chip, normalise inside the kernel that sums the K slices; larger ones run ttmi_gemm followed by
  * ttmi_add_bias_layer_norm.  Either `residual` (same dtype as out) or the pair residual_f32 / out_f32 (the
  * fp32 residual stream of ttmi_add_bias_layer_norm_residual32, which may alias each other) is given; the
- * unused ones are NULL.  a, w, out are densely packed (lda = ldb = k, ldc = n). */
+ * unused ones are NULL.  `out` must not alias `residual` or `a` (large problems store the bare product to `out`
+ * before the residual is read); a call that passes the same buffer is refused.  a, w, out are densely packed
+ * (lda = ldb = k, ldc = n). */
 TTMI_API int ttmi_gemm_bias_layer_norm(const void* a, const void* w, void* out, const void* residual,
                                        const float* residual_f32, const void* bias, const void* gamma,
                                        const void* beta, float* out_f32, int64_t m, int64_t n, int64_t k, float eps,
                                        int dtype, void* stream);
+
+/* ttmi_gemm_bias_layer_norm for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * arguments, same kernels and bit-identical results; the fp32 partial tiles of a product that is cut along K
+ * live in a buffer of TTMI_STATIC_SCRATCH_BYTES that is part of the library's device image (every GPU the
+ * library runs on holds it until the process ends) instead of the per-stream workspace ttmi_gemm_bias_layer_norm
+ * allocates on first use.  The call reaches no hipMalloc / hipFree.  A problem whose K slices need more than
+ * that buffer (slices * m * n * 4 bytes; m = 2560, n = 768, k = 3072 in four slices is the largest the encoder
+ * configurations produce) is refused with TTMI_EINVAL; problems large enough to run unsplit need no scratch
+ * and are accepted at any size.  Nothing has to be cleared between calls (every partial tile that is read
+ * has been written by the same call), but all calls on one GPU share the buffer: calls that overlap in time
+ * on one GPU (different streams or threads) race. */
+#define TTMI_STATIC_SCRATCH_BYTES (32u << 20)
+TTMI_API int ttmi_gemm_bias_layer_norm_static(const void* a, const void* w, void* out, const void* residual,
+                                              const float* residual_f32, const void* bias, const void* gamma,
+                                              const void* beta, float* out_f32, int64_t m, int64_t n, int64_t k,
+                                              float eps, int dtype, void* stream);
 
 /* kernels::AddBiasAct<T, Act>  (layers/kernels/activation.cpp:33-55, 90-119).
  * out[m,n] = act(out[m,n] + bias[n]) in place; gelu is the tanh form. */

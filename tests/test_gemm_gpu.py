@@ -88,6 +88,57 @@ def test_fused_epilogues_small_m_long_k(ttmi, oracle, dt):
     assert max_abs(host(C), base + rounded(bias, dt) + rounded(res, dt)) <= GEMM_TOL[dt] * 3
 
 
+@pytest.fixture
+def large_tile_forced():
+    """TTMI_LARGE_TILE=1 sends every eligible problem to the one-wavefront-per-SIMD kernel whatever its size."""
+    import os
+    old = os.environ.get("TTMI_LARGE_TILE")
+    os.environ["TTMI_LARGE_TILE"] = "1"
+    yield
+    if old is None:
+        del os.environ["TTMI_LARGE_TILE"]
+    else:
+        os.environ["TTMI_LARGE_TILE"] = old
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(256, 192, 128), (1, 8, 128), (300, 200, 256), (777, 776, 384), (2560, 768, 768),
+                                   (515, 3072, 256), (4100, 1000, 128), (64, 2304, 768)])
+def test_large_tile_kernel_against_oracle_and_small_tiles(ttmi, oracle, large_tile_forced, dt, M, N, K):
+    """The 256 x 192 tile kernel (four wavefronts, accumulators in AGPRs) on whole, ragged and tiny problems: plain
+    product, bias, bias + GELU.  Bound as for any MatMul against the oracle; the plain and the bias form must also
+    give the bits of the 8-wavefront kernels (same sums in the same order, same rounding)."""
+    import ctypes
+    import os
+    rng = np.random.default_rng(M + N + K)
+    A, W = _ab(rng, M, N, K, 1)
+    bias = rng.standard_normal(N).astype(np.float32)
+    dA, dW, db = dev(A, dt), dev(W, dt), dev(bias, dt)
+    base = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+
+    def run(epilogue):
+        C = torch.full((M, N), float("nan"), dtype=dA.dtype, device="cuda")
+        if epilogue is None:
+            ok(ttmi.ttmi_gemm(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, 1, 1.0, 0.0, TTMI_DTYPES[dt], stream()))
+        elif epilogue == "bias":
+            ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, capi.EPI_BIAS, ctypes.byref(_epi(bias=db)),
+                                    TTMI_DTYPES[dt], stream()))
+        else:
+            ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, capi.EPI_BIAS_ACT,
+                                    ctypes.byref(_epi(bias=db, act=capi.ACT_GELU)), TTMI_DTYPES[dt], stream()))
+        torch.cuda.synchronize()
+        return C
+
+    got = {e: run(e) for e in (None, "bias", "gelu")}
+    assert max_abs(host(got[None]), base) <= GEMM_TOL[dt]
+    assert max_abs(host(got["bias"]), base + rounded(bias, dt)) <= GEMM_TOL[dt] * 3
+    assert max_abs(host(got["gelu"]), oracle.add_bias_act(base, rounded(bias, dt), 0)) <= GEMM_TOL[dt] * 3
+    if (M, N, K) != (64, 2304, 768):  # that one is cut along K by the other path: another summation order
+        os.environ["TTMI_LARGE_TILE"] = "0"
+        assert torch.equal(run(None), got[None])
+        assert torch.equal(run("bias"), got["bias"])
+
+
 LN_TOL = {"f32": 1e-4, "f16": 4e-3, "bf16": 3e-2}  # relative to 1 + |expected|; large shapes round the product to 16 bits first
 
 

@@ -1,6 +1,7 @@
 // C ABI of the MFMA GEMM family: argument checks, epilogue selection and the static scratch buffer.
 // The kernels, epilogues and launch heuristics live in gemm_impl.h.
 #include "gemm_impl.h"
+#include "gemm_w4.h"
 
 namespace ttmi {
 

@@ -1226,25 +1226,36 @@ struct TileConfig {
 };
 constexpr TileConfig kTileConfigs[] = {
     {256, 256, 1, 1.00f}, {256, 192, 1, 0.93f}, {256, 128, 1, 0.82f}, {128, 128, 2, 0.62f}, {64, 64, 4, 0.30f}};
-constexpr int kNumCus = 256;
 
-static int pick_tile(int64_t m, int64_t n, int64_t batch) {
+static double tile_cost(const TileConfig& c, int64_t m, int64_t n, int64_t batch) {
+  const int64_t tiles = ceil_div(m, c.bm) * ceil_div(n, c.bn) * batch;
+  const int64_t slots = (int64_t)compute_units() * c.per_cu;
+  const int64_t full = tiles / slots, rem = tiles % slots;
+  const double t = (double)c.bm * c.bn / c.eff;
+  return (double)full * c.per_cu * t + (double)ceil_div(rem, compute_units()) * t;
+}
+
+static int pick_tile(int64_t m, int64_t n, int64_t batch, double* cost_out = nullptr) {
   int best = 0;
   double best_cost = 1e300;
   for (int i = 0; i < (int)(sizeof(kTileConfigs) / sizeof(kTileConfigs[0])); ++i) {
-    const TileConfig& c = kTileConfigs[i];
-    const int64_t tiles = ceil_div(m, c.bm) * ceil_div(n, c.bn) * batch;
-    const int64_t slots = (int64_t)kNumCus * c.per_cu;
-    const int64_t full = tiles / slots, rem = tiles % slots;
-    const double t = (double)c.bm * c.bn / c.eff;
-    const double cost = (double)full * c.per_cu * t + (double)ceil_div(rem, kNumCus) * t;
+    const double cost = tile_cost(kTileConfigs[i], m, n, batch);
     if (cost < best_cost) {
       best_cost = cost;
       best = i;
     }
   }
+  if (cost_out != nullptr) *cost_out = best_cost;
   return best;
 }
+
+// Hook for the one-wavefront-per-SIMD kernel of gemm_w4.h, which specialises it for the element types and
+// epilogues it serves: wanted() says whether that kernel should take the problem, launch() runs it.
+template <typename T, typename Epi, typename Enable = void>
+struct LargeTileKernel {
+  static bool wanted(const GemmArgs&, const Epi&, int, bool) { return false; }
+  static int launch(const GemmArgs&, const Epi&, hipStream_t) { return 0; }
+};
 
 // Whether (and how) a problem on the [N,K]-weights path is cut along K.
 enum class SplitKind { kNone, kSmallTiles, kDmaTiles };
@@ -1281,6 +1292,7 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
     if (aligned && g.k % BK == 0) {
       bool column_pass = false;
       if constexpr (HasColumnPass<Epi>::value) column_pass = epi.v_pitch > 0;
+      if (LargeTileKernel<T, Epi>::wanted(g, epi, batch, aligned)) return LargeTileKernel<T, Epi>::launch(g, epi, s);
       switch (pick_tile(g.m, g.n, batch)) {
         case 0: return launch_fast<T, 256, 256, 2, 4, Epi>(g, epi, batch, s);
         case 1: return launch_fast<T, 256, 192, 4, 2, Epi>(g, epi, batch, s);

@@ -1,0 +1,528 @@
+// Large-tile GEMM kernel for gfx950: one wavefront per SIMD, accumulators in the AGPR half of the
+// register file, 16-bit operands and outputs.
+//
+//   C[M,N] = epilogue(A[M,K] * B[N,K]^T)   (both operands K-contiguous, 16-byte aligned, K a multiple of 128 elements)
+//
+// A workgroup of four wavefronts (2 x 2) owns a 256 x BN tile (BN = 256 or 192); each wavefront owns
+// 128 x BN/2 of it: 256 (192) fp32 accumulators per lane, which only fit because a lone wavefront on a
+// SIMD may use all 512 registers of a lane.  Per 16 bytes of K a wavefront then reads 0.5 (0.58) LDS
+// operand fragments per 32x32 MFMA instead of the 0.75 of the 8-wavefront tiling.
+//
+// K advances in steps of 128 bytes per row through a two-stage LDS ring filled by
+// `buffer_load_dwordx4 ... lds` DMA loads (no VGPR staging).  The workgroup is persistent: it walks a
+// list of tiles, and the sequence of (tile, K step) pairs is one flat stream, so that the DMA runs two K
+// steps ahead of the MFMAs also across tile boundaries and a tile's epilogue runs with the next tile's
+// first K steps already landing in LDS.  The instruction order of a K step is written out MFMA by MFMA
+// (LDS reads and DMA loads at fixed slots between the MFMAs, a scheduling fence after each): what
+// limits the K loop is how evenly the DMA loads reach the memory pipeline and how long they have to land
+// before the stage barrier, not the LDS or the matrix pipe.
+//
+// The MFMA operands are swapped (the weight fragment is the matrix instruction's A operand), which leaves
+// every lane with runs of four consecutive COLUMNS of one output row; one v_permlane32_swap per register
+// pairs lanes up so that a lane holds eight consecutive columns.  Bias and activation are applied there,
+// the eight values are rounded to the output type and staged, 32 rows at a time, in a strip of LDS private
+// to the wavefront (no workgroup barrier), from which they leave as whole 256-byte row segments; stores
+// straight from the accumulator layout would touch 32 different rows per instruction.  Epilogues with a
+// column pass (V kept transposed by the QKV split) run the tiles of that column range unswapped: a lane
+// then holds eight consecutive ROWS of one column, which is what store_col8 wants.
+#pragma once
+
+#include <cstdlib>
+
+#include "gemm_impl.h"
+
+namespace ttmi {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+// 16 bytes in flight between a global load and its LDS write: a first-class vector value, so that arrays of it
+// are promoted to registers.
+typedef uint32_t __attribute__((ext_vector_type(4), may_alias)) Quad;
+template <int V>
+using template_int = std::integral_constant<int, V>;
+
+// One MF x MF block of the output: the matrix instruction and its accumulator.
+template <typename T, int MF>
+struct MmaBlock;
+template <>
+struct MmaBlock<f16, 32> {
+  using Acc = floatx16;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct MmaBlock<bf16, 32> {
+  using Acc = floatx16;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct MmaBlock<int8_t, 32> {
+  using Acc = intx16;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct MmaBlock<f16, 16> {
+  using Acc = floatx4;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct MmaBlock<bf16, 16> {
+  using Acc = floatx4;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct MmaBlock<int8_t, 16> {
+  using Acc = intx4;
+  static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), c, 0, 0, 0);
+  }
+};
+
+// Lanes of the lower half of each lane pair (MF = 32: lanes 0..31 with 32..63; MF = 16: 16-lane rows 0 with 1,
+// 2 with 3) keep `a` and receive the partner's `a` in `b`; the upper ones keep `b` and receive the partner's `b`
+// in `a`.  Afterwards {a, b} of every lane are neighbours in the output.
+template <int MF, typename S>
+__device__ __forceinline__ void pair_swap(S& a, S& b) {
+  static_assert(sizeof(S) == 4, "one register");
+#if defined(__HIP_DEVICE_COMPILE__)
+  const unsigned ua = __builtin_bit_cast(unsigned, a), ub = __builtin_bit_cast(unsigned, b);
+  if constexpr (MF == 32) {
+    const auto r = __builtin_amdgcn_permlane32_swap(ua, ub, false, false);
+    a = __builtin_bit_cast(S, (unsigned)r[0]);
+    b = __builtin_bit_cast(S, (unsigned)r[1]);
+  } else {
+    const auto r = __builtin_amdgcn_permlane16_swap(ua, ub, false, false);
+    a = __builtin_bit_cast(S, (unsigned)r[0]);
+    b = __builtin_bit_cast(S, (unsigned)r[1]);
+  }
+#endif
+}
+
+// Bias of eight consecutive columns, kept in storage precision (16 bytes for 2-byte types) until it is added.
+template <typename BT>
+struct BiasVec {
+  static constexpr int kPer = 16 / sizeof(BT), kChunksPerVec = 8 / kPer;
+  Chunk raw[kChunksPerVec];
+  bool present;
+  __device__ __forceinline__ void load(const BT* bias, int ncol) {
+    present = bias != nullptr;
+    if (present) {
+#pragma unroll
+      for (int c = 0; c < kChunksPerVec; ++c) raw[c] = *reinterpret_cast<const Chunk*>(bias + ncol + c * kPer);
+    }
+  }
+  template <typename S>
+  __device__ __forceinline__ void add_to(S (&out)[8]) const {
+    if (!present) return;
+#pragma unroll
+    for (int c = 0; c < kChunksPerVec; ++c) {
+      const Vec<BT, kPer> v = __builtin_bit_cast(Vec<BT, kPer>, raw[c]);
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) out[c * kPer + e] += (S)to_float(v.v[e]);
+    }
+  }
+};
+
+constexpr int kW4Threads = 256;
+
+// LDS of the kernel: two K-loop stages plus one private epilogue strip per wavefront (MF rows x BN/2 columns of
+// the 2-byte output type; rows padded by 16 bytes when that does not fit a power-of-two swizzle).
+template <int BN, int MF>
+constexpr int w4_strip_pitch() { return BN == 256 ? 256 : BN + 16; }  // bytes per staged row (BN/2 columns of 2 bytes)
+template <int BN, int MF>
+constexpr int w4_lds_bytes() { return 2 * (256 + BN) * kRowBytes + 4 * MF * w4_strip_pitch<BN, MF>(); }
+
+// What the kernel needs from an epilogue besides bias_ptr(): finish(x) applied to acc + bias in fp32, and
+// dest8(m, n), the address of the 16 bytes that hold columns n..n+7 of output row m.
+template <typename T, int BN, int MF, typename Epi>
+__global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, const Epi epi) {
+  static_assert(sizeof(T) == 2, "16-bit operands");
+  constexpr int BM = 256;
+  constexpr int BK = kRowBytes / sizeof(T);
+  constexpr int RB = 128 / MF, CB = BN / 2 / MF;   // blocks per wavefront: rows, columns
+  constexpr int SUB = MF == 32 ? 4 : 2;            // K substeps per 128-byte K step
+  constexpr int CPS = kChunks / SUB;               // 16-byte chunks of a row per substep; lane / MF picks one
+  constexpr int ACC = MF * MF / kWave;             // accumulator registers per block
+  constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_LOADS = BM / 8 / 4, B_LOADS = BN / 8 / 4;  // 16-byte loads per lane and K step
+  constexpr int LOADS = A_LOADS + B_LOADS;
+  constexpr int PITCH = w4_strip_pitch<BN, MF>(), CPR = BN / 2 / 8;  // staged row: bytes, 16-byte chunks
+  constexpr bool XOR_STRIP = (CPR & (CPR - 1)) == 0;
+  static_assert(BN % (2 * MF) == 0 && BN % 32 == 0, "tile width");
+  static_assert(CB % 2 == 0 || MF == 32, "16-wide blocks are stored in pairs");
+  static_assert(A_LOADS % 2 == 0 && B_LOADS % 2 == 0, "the LDS swizzle of a load depends on its parity only");
+  using MB = MmaBlock<T, MF>;
+  using Acc = typename MB::Acc;
+
+  extern __shared__ __align__(16) char smem[];
+
+  // Tiles of this workgroup: XCD x owns [x*per_xcd, (x+1)*per_xcd); its workgroups stride through it together.
+  const int tiles = g.tiles_m * g.tiles_n;
+  const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
+  const int xcd = (int)(blockIdx.x % kNumXcd), stride = (int)(gridDim.x / kNumXcd);
+  const int xcd_end = min((xcd + 1) * per_xcd, tiles);
+  const int first = xcd * per_xcd + (int)(blockIdx.x / kNumXcd);
+  if (first >= xcd_end) return;
+  const int my_tiles = (xcd_end - first + stride - 1) / stride;
+  const int ksteps = g.k / BK;  // even (checked by the launcher)
+  const int total_steps = my_tiles * ksteps;
+
+  const int64_t lda_bytes = g.lda * (int64_t)sizeof(T), ldb_bytes = g.ldb * (int64_t)sizeof(T);
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm0 = (wave / 2) * 128, wn0 = (wave % 2) * (BN / 2);
+  const int lrow = lane % MF, lgrp = lane / MF;
+  // LDS: [A stage 0][A stage 1][B stage 0][B stage 1][epilogue strips]; the stage of an operand is an immediate offset
+  const int a_row0 = (wm0 + lrow) * kRowBytes, b_row0 = 2 * A_BYTES + (wn0 + lrow) * kRowBytes;
+  const int swz = (lrow >> 1) & 7;
+
+  // ---- DMA cursor.  `buffer_load_dwordx4 ... lds` copies 8 tile rows (64 lanes x 16 bytes) straight into LDS; the
+  //      LDS side is linear in the lane id, so the XOR swizzle is applied on the global side: lane l fills physical
+  //      chunk l%8 of row l/8 and therefore fetches logical chunk (l%8) ^ ((row>>1)&7).  The LOADS loads of one K
+  //      step are not issued as a burst: the memory pipeline takes about 20 cycles per load and serves the four
+  //      wavefronts in turn, and a wavefront that finds its queue full stops issuing MFMAs.
+  int dma_step = 0, dma_k = 0, dma_tile = first;
+  uint32_t voa[A_LOADS], vob[B_LOADS];  // per-lane byte offsets from the tile's first row (row clamp and swizzle inside)
+  uint32_t a_soff = 0, b_soff = 0;  // byte offset of the cursor's tile in A and in B (matrices below 2 GiB, checked by the launcher)
+  auto dma_point = [&](int tile) __attribute__((always_inline)) {
+    int tile_m, tile_n;
+    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int sub = lane >> 3, p = lane & 7;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int row = (wave * A_LOADS + i) * 8 + sub;
+      voa[i] = (uint32_t)(min(m0 + row, g.m - 1) - m0) * (uint32_t)lda_bytes + ((p ^ ((row >> 1) & 7)) << 4);
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const int row = (wave * B_LOADS + i) * 8 + sub;
+      vob[i] = (uint32_t)(min(n0 + row, g.n - 1) - n0) * (uint32_t)ldb_bytes + ((p ^ ((row >> 1) & 7)) << 4);
+    }
+    a_soff = (uint32_t)m0 * (uint32_t)lda_bytes;
+    b_soff = (uint32_t)n0 * (uint32_t)ldb_bytes;
+  };
+  // load i of K step `dma_step` into stage dma_step & 1
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef __attribute__((address_space(3))) char lds_char;
+  lds_char* lds0 = reinterpret_cast<lds_char*>(reinterpret_cast<uintptr_t>(smem));
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(g.a), 0, (int)min((int64_t)g.m * lda_bytes, (int64_t)0x7fffffff), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(g.b), 0, (int)min((int64_t)g.n * ldb_bytes, (int64_t)0x7fffffff), 0x00020000);
+  auto dma_issue_one = [&](int i) __attribute__((always_inline)) {
+    if (i < A_LOADS) {
+      lds_char* as = lds0 + (dma_step & 1) * A_BYTES + wave * (A_LOADS * 1024);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, as + i * 1024, 16, voa[i], a_soff + dma_k * kRowBytes, 0, 0);
+    } else {
+      lds_char* bs = lds0 + 2 * A_BYTES + (dma_step & 1) * B_BYTES + wave * (B_LOADS * 1024);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, bs + (i - A_LOADS) * 1024, 16, vob[i - A_LOADS], b_soff + dma_k * kRowBytes, 0, 0);
+    }
+  };
+#else
+  auto dma_issue_one = [&](int) {};
+#endif
+  auto dma_issue = [&](auto lo_tag, auto hi_tag) __attribute__((always_inline)) {
+    constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
+#pragma unroll
+    for (int i = LO; i < HI; ++i) dma_issue_one(i);
+  };
+  // Move the cursor to the next K step of the flat sequence.  Past its end it stays on the last step: the surplus
+  // loads at the end of the kernel re-fetch that step into stages nobody reads any more.
+  auto dma_advance = [&]() __attribute__((always_inline)) {
+    ++dma_step;
+    if (dma_step < total_steps && ++dma_k == ksteps) {
+      dma_k = 0;
+      dma_tile += stride;
+      dma_point(dma_tile);
+    }
+  };
+
+  Chunk fa[2][RB], fb[2][CB];
+  auto read_frags = [&](int stage, int sub, Chunk (&a)[RB], Chunk (&b)[CB]) __attribute__((always_inline)) {
+    const int off = ((sub * CPS + lgrp) ^ swz) << 4;
+#pragma unroll
+    for (int i = 0; i < RB; ++i) a[i] = *reinterpret_cast<const Chunk*>(smem + (a_row0 + off) + (stage * A_BYTES + i * MF * kRowBytes));
+#pragma unroll
+    for (int j = 0; j < CB; ++j) b[j] = *reinterpret_cast<const Chunk*>(smem + (b_row0 + off) + (stage * B_BYTES + j * MF * kRowBytes));
+  };
+
+  Acc acc[RB][CB];
+  // SWAP: the weight fragment is the instruction's A operand -> a lane owns one output ROW of a block.
+  // One substep in exact instruction order: MFMA m of this substep, then LDS read m of the next one (m < READS, so
+  // the reads have landed long before their use and before the barrier), then a DMA load when m is one of NL evenly
+  // spaced slots (the memory pipeline takes about 20 cycles per DMA load and serves the four wavefronts in turn: a
+  // wavefront that issues them faster than one per three MFMAs blocks at the queue with the matrix pipe idle).
+  // A scheduling fence after every MFMA keeps the compiler from regrouping them.
+  // rd_stage/rd_sub: what the reads fetch; DLO: index of the first DMA load issued here.
+  constexpr int READS = RB + CB, MMAS = RB * CB;
+  auto substep = [&](auto swap_tag, auto cur_tag, auto rd_stage_tag, auto rd_sub_tag, auto dlo_tag, auto nl_tag, auto ext_tag) __attribute__((always_inline)) {
+    constexpr bool SWAP = decltype(swap_tag)::value;
+    constexpr int CUR = decltype(cur_tag)::value, RS = decltype(rd_stage_tag)::value, RSUB = decltype(rd_sub_tag)::value;
+    constexpr int DLO = decltype(dlo_tag)::value, NL = decltype(nl_tag)::value, EXT = decltype(ext_tag)::value;  // NL loads over the first EXT MFMAs
+    static_assert(NL <= EXT && EXT <= MMAS, "at most one DMA load per MFMA");
+    const int off = ((RSUB * CPS + lgrp) ^ swz) << 4;
+#pragma unroll
+    for (int m = 0; m < MMAS; ++m) {
+      const int i = m / CB, j = m % CB;
+      if constexpr (SWAP) MB::run(fb[CUR][j], fa[CUR][i], acc[i][j]);
+      else MB::run(fa[CUR][i], fb[CUR][j], acc[i][j]);
+      if (m < RB) fa[CUR ^ 1][m] = *reinterpret_cast<const Chunk*>(smem + (a_row0 + off) + (RS * A_BYTES + m * MF * kRowBytes));
+      else if (m < READS) fb[CUR ^ 1][m - RB] = *reinterpret_cast<const Chunk*>(smem + (b_row0 + off) + (RS * B_BYTES + (m - RB) * MF * kRowBytes));
+      if (NL > 0 && m < EXT && ((m + 1) * NL) / EXT != (m * NL) / EXT) dma_issue_one(DLO + (m * NL) / EXT);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // How the LOADS loads of one K step are spread: D3 behind the barrier of step s, D0 and D1 in the first two
+  // substeps of step s+1; the substep in front of the barrier issues none, so that every load has at least a
+  // substep to land.  (SUB = 2: the barrier sits between the two substeps and all loads follow it.)
+  constexpr int D3 = SUB == 4 ? LOADS / 2 : LOADS;
+  constexpr int D0 = SUB == 4 ? LOADS - D3 : 0;
+  constexpr int D1 = 0;
+  constexpr int EXT1 = 1;
+  static_assert(D3 + D0 + D1 == LOADS && D3 >= 0, "every load of a K step is issued once");
+  template_int<0> I0;
+
+  // One K step.  P = parity of the step = its LDS stage.
+  auto k_step = [&](auto parity_tag, auto swap_tag) __attribute__((always_inline)) {
+    constexpr int P = decltype(parity_tag)::value;
+    if constexpr (SUB == 4) {
+      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<1>{}, template_int<D3>{}, template_int<D0>{}, template_int<MMAS>{});
+      substep(swap_tag, template_int<1>{}, template_int<P>{}, template_int<2>{}, template_int<D3 + D0>{}, template_int<D1>{}, template_int<EXT1>{});
+      dma_advance();
+      __builtin_amdgcn_sched_barrier(0);
+      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<3>{}, I0, I0, template_int<MMAS>{});
+    } else {
+      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<1>{}, I0, I0, template_int<MMAS>{});
+      dma_advance();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // everyone has read all of this stage (the last reads were issued half a substep ago); the other stage has landed
+    dma_landed_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    substep(swap_tag, template_int<1>{}, template_int<P ^ 1>{}, template_int<0>{}, I0, template_int<D3>{}, template_int<MMAS>{});
+  };
+
+  // ---- prologue: K step 0 lands, the first loads of K step 1 are under way ----
+  dma_point(dma_tile);
+  dma_issue(std::integral_constant<int, 0>{}, std::integral_constant<int, LOADS>{});
+  dma_advance();
+  dma_landed_barrier();
+  dma_issue(std::integral_constant<int, 0>{}, std::integral_constant<int, D3>{});
+  read_frags(0, 0, fa[0], fb[0]);
+
+  char* strip = smem + 2 * STAGE + wave * (MF * PITCH);
+  int tile = first;
+  for (int t = 0; t < my_tiles; ++t, tile += stride) {
+    int tile_m, tile_n;
+    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    bool swap = true;
+    if constexpr (HasColumnPass<Epi>::value) swap = !(epi.column_pass() && n0 >= epi.first_column_of_pass());
+
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int j = 0; j < CB; ++j)
+#pragma unroll
+        for (int e = 0; e < ACC; ++e) acc[i][j][e] = 0;
+
+    const auto* bias = epi.bias_ptr();
+    using BiasT = typename std::remove_cv<typename std::remove_pointer<decltype(bias)>::type>::type;
+    const int m_lim = g.m, n_lim = g.n;
+    if (swap) {
+      for (int kt = 0; kt < ksteps; kt += 2) {
+        k_step(std::integral_constant<int, 0>{}, std::true_type{});
+        k_step(std::integral_constant<int, 1>{}, std::true_type{});
+      }
+      // A lane now owns, per block (pair), eight consecutive columns of one row: + bias, finish(), round to T,
+      // 16 bytes into the wavefront's strip; the strip goes out row-contiguous, 16 bytes per lane.
+      constexpr int NV = MF == 32 ? CB * 2 : CB / 2;
+      BiasVec<BiasT> bv[NV];
+      int chunk_of[NV];
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        if constexpr (MF == 32) chunk_of[v] = (v / 2) * 4 + (v % 2) * 2 + lgrp;
+        else chunk_of[v] = 2 * (2 * v + (lgrp & 1)) + (lgrp >> 1);
+        bv[v].load(bias, min(n0 + wn0 + chunk_of[v] * 8, n_lim - 8));  // N % 8 == 0
+      }
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+          float out[8];
+          if constexpr (MF == 32) {
+            const int j = v / 2, gp = v % 2;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float a = acc[i][j][8 * gp + e], b = acc[i][j][8 * gp + 4 + e];
+              pair_swap<32>(a, b);
+              out[e] = a;
+              out[4 + e] = b;
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float a = acc[i][2 * v][e], b = acc[i][2 * v + 1][e];
+              pair_swap<16>(a, b);
+              out[e] = a;
+              out[4 + e] = b;
+            }
+          }
+          {
+            // the bias stays packed between uses: widened once per strip it would occupy 64 registers across the
+            // whole epilogue (the asm statement keeps the compiler from hoisting the conversion out of the strip loop)
+            BiasVec<BiasT> b = bv[v];
+            asm volatile("" : "+v"(b.raw[0].w[0]), "+v"(b.raw[0].w[1]), "+v"(b.raw[0].w[2]), "+v"(b.raw[0].w[3]));
+            b.add_to(out);
+          }
+          T packed[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) packed[e] = from_float<T>(epi.finish(out[e]));
+          const int pc = XOR_STRIP ? (chunk_of[v] ^ (lrow & (CPR - 1))) : chunk_of[v];
+          *reinterpret_cast<Chunk*>(strip + lrow * PITCH + (pc << 4)) = pack_chunk(packed);
+          __builtin_amdgcn_sched_barrier(0);  // one group of eight at a time: no wholesale hoisting of accumulator reads
+        }
+        // same wavefront, LDS operations complete in order: no barrier between the writes and the reads
+        constexpr int PASSES = (MF * CPR + kWave - 1) / kWave;
+#pragma unroll
+        for (int pass = 0; pass < PASSES; ++pass) {
+          const int idx = pass * kWave + lane;
+          const int r = idx / CPR, c = idx % CPR;
+          if (MF * CPR % kWave != 0 && r >= MF) continue;
+          const int pc = XOR_STRIP ? (c ^ (r & (CPR - 1))) : c;
+          const Chunk x = *reinterpret_cast<const Chunk*>(strip + r * PITCH + (pc << 4));
+          const int m = m0 + wm0 + i * MF + r, ncol = n0 + wn0 + c * 8;
+          if (m < m_lim && ncol < n_lim) *reinterpret_cast<Chunk*>(epi.dest8(m, ncol)) = x;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      if constexpr (HasColumnPass<Epi>::value) {
+        for (int kt = 0; kt < ksteps; kt += 2) {
+          k_step(std::integral_constant<int, 0>{}, std::false_type{});
+          k_step(std::integral_constant<int, 1>{}, std::false_type{});
+        }
+        // a lane owns column lrow of every block and, after the pair swap, eight consecutive rows of it
+        float bj[CB];
+        load_bias_columns_stride<CB, MF>(epi, n0 + wn0 + lrow, n_lim, bj);
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+          const int ncol = n0 + wn0 + j * MF + lrow;
+          if constexpr (MF == 32) {
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+#pragma unroll
+              for (int gp = 0; gp < 2; ++gp) {
+                float out[8];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  float a = acc[i][j][8 * gp + e], b = acc[i][j][8 * gp + 4 + e];
+                  pair_swap<32>(a, b);
+                  out[e] = a + bj[j];
+                  out[4 + e] = b + bj[j];
+                }
+                const int m = m0 + wm0 + i * 32 + 16 * gp + 8 * lgrp;
+                if (m < m_lim && ncol < n_lim) epi.store_col8(m, m_lim, ncol, out);
+              }
+          } else {
+#pragma unroll
+            for (int i = 0; i < RB; i += 2) {
+              float out[8];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                float a = acc[i][j][e], b = acc[i + 1][j][e];
+                pair_swap<16>(a, b);
+                out[e] = a + bj[j];
+                out[4 + e] = b + bj[j];
+              }
+              const int m = m0 + wm0 + (i + (lgrp & 1)) * 16 + 8 * (lgrp >> 1);
+              if (m < m_lim && ncol < n_lim) epi.store_col8(m, m_lim, ncol, out);
+            }
+          }
+        }
+      }
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // surplus DMA loads have landed before the LDS is given back
+}
+
+// Whether a problem may take this kernel: 16-bit type, one problem, aligned operands, an even number of K steps,
+// columns in groups of eight, operands below 2 GiB (32-bit buffer offsets).
+template <typename T>
+static bool w4_eligible(const GemmArgs& g, int batch, bool aligned) {
+  if (sizeof(T) != 2 || batch != 1 || !aligned || g.k_chunk != 0) return false;
+  constexpr int BK = kRowBytes / (int)sizeof(T);
+  if (g.k % (2 * BK) != 0 || g.n % 8 != 0) return false;
+  const int64_t limit = (int64_t)1 << 31;
+  return (int64_t)g.m * g.lda * (int64_t)sizeof(T) < limit && (int64_t)g.n * g.ldb * (int64_t)sizeof(T) < limit;
+}
+
+template <typename T, int BN, typename Epi>
+static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s) {
+  constexpr int LDS = w4_lds_bytes<BN, 32>();
+  static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
+  g.tiles_m = (g.m + 255) / 256;
+  g.tiles_n = (g.n + BN - 1) / BN;
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  TTMI_REQUIRE(tiles < (1ll << 30), "GEMM grid too large");
+  // one persistent workgroup per CU (the LDS allows no second one), a multiple of the XCD count
+  const unsigned grid = (unsigned)(std::min<int64_t>(ceil_div(tiles, kNumXcd), std::max(1, compute_units() / kNumXcd)) * kNumXcd);
+  auto kern = gemm_w4_kernel<T, BN, 32, Epi>;
+  const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
+  if (rc != 0) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kW4Threads), LDS, s, g, epi);
+  return launch_status("gemm_w4_kernel");
+}
+
+// The 256 x 192 tile against the tile configurations of the 8-wavefront kernels: the same cost model, with the
+// efficiency this kernel measured against them on the encoder shapes.
+constexpr TileConfig kW4Tile192{256, 192, 1, 1.06f};
+
+// TTMI_LARGE_TILE=0 keeps every problem on the 8-wavefront kernels, =1 sends every eligible problem here whatever
+// the cost model says (for A/B timing and for tests of small and ragged shapes); unset: the cost model decides.
+template <typename T, typename Epi>
+static bool w4_wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
+  if (!epi.vec || !w4_eligible<T>(g, batch, aligned)) return false;
+  if (const char* force = std::getenv("TTMI_LARGE_TILE")) {
+    if (force[0] == '0') return false;
+    if (force[0] == '1') return true;
+  }
+  double other = 0;
+  (void)pick_tile(g.m, g.n, batch, &other);
+  return tile_cost(kW4Tile192, g.m, g.n, batch) < other;
+}
+
+// Bias, and bias + activation.  With an activation the epilogue is a long stretch of VALU work (two transcendentals
+// per element) that nothing overlaps when a SIMD holds a single wavefront: inside the encoder the FFN1 product
+// (N = 3072, K = 768: twelve K steps per tile) ran 2.6 % slower here than on the 8-wavefront kernel, so those
+// problems come here only when forced.
+template <typename T, int ACT, bool HAS_ACT>
+struct LargeTileKernel<T, EpiBias<T, ACT, HAS_ACT, false>, typename std::enable_if<sizeof(T) == 2>::type> {
+  using Epi = EpiBias<T, ACT, HAS_ACT, false>;
+  static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
+    if (HAS_ACT) {
+      const char* force = std::getenv("TTMI_LARGE_TILE");
+      if (force == nullptr || force[0] != '1') return false;
+    }
+    return w4_wanted<T>(g, epi, batch, aligned);
+  }
+  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
+};
+template <typename T>
+struct LargeTileKernel<T, EpiAlphaBeta<T>, typename std::enable_if<sizeof(T) == 2>::type> {
+  using Epi = EpiAlphaBeta<T>;
+  static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
+    return epi.beta == 0.f && w4_wanted<T>(g, epi, batch, aligned);
+  }
+  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
+};
+
+}  // namespace ttmi

@@ -172,3 +172,53 @@ def test_converter_writes_the_reference_key_scheme(tmp_path):
     assert np.array_equal(got["pooler.dense.weight"], sd["pooler.dense.weight"].T)
     assert np.array_equal(got["embeddings.word_embeddings.weight"], sd["embeddings.word_embeddings.weight"])
 
+
+
+def _stored_npz(path, members):
+    """A zip archive of stored (uncompressed) members with the given raw bytes."""
+    import zipfile
+    with zipfile.ZipFile(path, "w", zipfile.ZIP_STORED) as z:
+        for name, raw in members.items():
+            z.writestr(name, raw)
+
+
+def _npy(header_text, payload=b""):
+    head = header_text.encode("latin1")
+    return b"\x93NUMPY\x01\x00" + len(head).to_bytes(2, "little") + head + payload
+
+
+@pytest.mark.parametrize("header", [
+    "{'descr': '<f4', 'fortran_order': False, 'shape': (2, 3), }",                # payload missing
+    "{'descr': '<f4', 'fortran_order': False, 'shape': (4611686018427387904, 4), }",  # product wraps around 2^64
+    "{'descr': '<f4', 'fortran_order': False, 'shape': (99999999999999999999999, ), }",
+    "{'descr': '<f4', 'fortran_order': False, 'shape' ",                          # no parenthesis
+    "{'descr': '<f4', 'fortran_order': False }",                                   # no shape
+    "{'descr': <f4, 'fortran_order': False, 'shape': (1, ), }",                    # unquoted dtype
+    "{'descr': '<fx', 'fortran_order': False, 'shape': (1, ), }",                  # dtype size is not a number
+    "{'descr'",                                                                    # nothing after the key
+    "{'descr': '<f4', 'fortran_order':",                                           # ends inside a value
+    "{'descr': '<f4', 'fortran_order': True, 'shape': (1, ), }",
+    "{'descr': '<c8', 'fortran_order': False, 'shape': (1, ), }",
+])
+def test_npz_reader_refuses_malformed_members(tmp_path, header):
+    """A malformed member ends in the loader's own error (RuntimeError), never in a crash or a C++ library exception
+    of another type; a well-formed neighbour is no excuse."""
+    import turbo_transformers.turbo_transformers_cxx as cxx
+    path = str(tmp_path / "m.npz")
+    _stored_npz(path, {"ok.npy": _npy("{'descr': '<f4', 'fortran_order': False, 'shape': (1, ), }".ljust(118) + "\n",
+                                      np.float32(1).tobytes()),
+                       "bad.npy": _npy(header.ljust(118) + "\n", b"\0" * 16)})
+    with pytest.raises(RuntimeError):
+        cxx.load_npz(path)
+
+
+def test_npz_reader_refuses_sizes_beyond_the_file(tmp_path):
+    import turbo_transformers.turbo_transformers_cxx as cxx
+    path = str(tmp_path / "m.npz")
+    np.savez(path, a=np.arange(4, dtype=np.float32))
+    data = bytearray(open(path, "rb").read())
+    cd = data.rfind(b"PK\x01\x02")
+    data[cd + 20:cd + 28] = (0x7ffffff0).to_bytes(4, "little") * 2  # compressed and uncompressed size of the member
+    open(path, "wb").write(bytes(data))
+    with pytest.raises(RuntimeError):
+        cxx.load_npz(path)

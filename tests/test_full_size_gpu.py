@@ -50,9 +50,11 @@ def full(request):
     mask = (np.arange(S)[None, :] < lens[:, None]).astype(np.int64)
     tmodel = tt.BertModel.from_torch(low, torch.device("cuda:0"), "turbo")
     d_ids, d_mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
-    out = tmodel(d_ids, attention_masks=d_mask)[0].clone()
+    res = tmodel(d_ids, attention_masks=d_mask, output_fp32_hidden_state=True)
+    out = res[0].clone()
+    out32 = res[-1].clone() if res[-1] is not None else None  # bfloat16 models: the unrounded final hidden state
     yield {"model": tmodel, "weights": weights, "ids": ids, "mask": mask, "lens": lens, "d_ids": d_ids, "d_mask": d_mask,
-           "out": out, "layers": layers, "heads": heads, "dtype": dtype, "sampled": sampled}
+           "out": out, "out32": out32, "layers": layers, "heads": heads, "dtype": dtype, "sampled": sampled}
     del tmodel, low
     torch.cuda.empty_cache()
 
@@ -69,14 +71,20 @@ def test_sampled_sequences_of_the_full_batch_match_the_oracle(full, oracle):
         ext = (-10000.0 * (1 - full["mask"][b])).astype(np.float32).reshape(1, 1, 1, S)
         want = oracle.bert_encoder(emb, ext, layers, full["heads"])[0]
         # rows under the mask are computed too (as the reference does) but nothing downstream reads them
-        err = np.abs(got[b, :n] - want[:n])
         if full["dtype"] == torch.float16:
-            assert err.max() < 2e-2, "sequence %d" % b
+            assert np.abs(got[b, :n] - want[:n]).max() < 2e-2, "sequence %d" % b
         else:
-            # a bfloat16 output carries half an ulp (2^-8 relative) of representation error whatever computed
-            # it; the bound applies to what exceeds that, as a quantile plus a cap over the 24 layers
-            excess = err - 2.0 ** -8 * np.abs(want[:n])
-            assert (excess > 2e-2).mean() <= 1e-4 and excess.max() < 3e-2, "sequence %d" % b
+            # bfloat16: the bound is on the unrounded (fp32) final hidden state the model hands out with the bfloat16
+            # tensor; the bfloat16 tensor is the rounding of it.  Through 24 layers the operand roundings that bfloat16 matrix
+            # products cannot avoid (LayerNorm output, attention context, GELU output, each rounded once before it
+            # enters a product, plus the 16-bit product in front of each LayerNorm) put the mean deviation at 3e-3 and
+            # the largest of the 200k values of a sequence at 0.020-0.025 (an emulation of exactly these roundings in
+            # float64 gives the same figures); so the bound at this depth is stated as: mean, all but 1e-5 of the
+            # values inside 2e-2, none outside 2.5e-2.
+            got32 = host(full["out32"][b])
+            err = np.abs(got32[:n] - want[:n])
+            assert err.mean() < 4e-3 and (err > 2e-2).mean() <= 1e-5 and err.max() < 2.5e-2, "sequence %d: %g" % (b, err.max())
+            assert np.array_equal(got[b], host(full["out32"][b].to(torch.bfloat16)))
 
 
 def test_permuting_the_batch_permutes_the_output_bit_for_bit(full):

@@ -167,12 +167,15 @@ __global__ __launch_bounds__(kBlock) void lookup_embedding_kernel(T* __restrict_
   const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   if (row >= num_ids) return;
   const int64_t id = ids[row];
+  T* dst = out + row * hidden;
   if (id < 0 || id >= vocab) {
+    // raise the flag the host reads at its next synchronisation, and leave NaN in the row: the buffer may be a
+    // recycled block, and whatever it held must not pass for an embedding
     if (threadIdx.x % kWave == 0) *err = 1;
+    for (int c = threadIdx.x % kWave; c < hidden; c += kWave) dst[c] = from_float<T>(__builtin_nanf(""));
     return;
   }
   const T* src = table + id * hidden;
-  T* dst = out + row * hidden;
   for (int c = (threadIdx.x % kWave) * VEC; c < hidden; c += kWave * VEC) {
     Vec<T, VEC> x = load_vec<T, VEC>(src + c);
     if (ADD) {
@@ -199,7 +202,12 @@ __global__ __launch_bounds__(kBlock) void bert_embedding_kernel(
   if (row >= num_ids) return;  // whole wavefront exits together
   const int64_t id = ids[row], p = pos_ids[row], tt = type_ids[row];
   if (id < 0 || id >= vocab || p < 0 || p >= max_pos || tt < 0 || tt >= num_types) {
+    // as in lookup_embedding_kernel: flag for the host, NaN in the row
     if (lane == 0) *err = 1;
+    for (int c = lane; c < hidden; c += kWave) {
+      out[row * hidden + c] = from_float<T>(__builtin_nanf(""));
+      if (out32) out32[row * hidden + c] = __builtin_nanf("");
+    }
     return;
   }
   const T* wrow = word + id * hidden;
@@ -230,7 +238,7 @@ __global__ __launch_bounds__(kBlock) void bert_embedding_kernel(
   sum = group_sum<kWave>(sum);
   sumsq = group_sum<kWave>(sumsq);
   const float mean = sum / (float)hidden;
-  const float var = sumsq / (float)hidden - mean * mean;
+  const float var = fmaxf(sumsq / (float)hidden - mean * mean, 0.f);  // cancellation on a near-constant row must not go negative
   const float rstd = 1.0f / sqrtf(var + eps);
   T* orow = out + row * hidden;
 #pragma unroll

@@ -788,7 +788,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_layer_norm_kernel(const flo
   sum = red[0][0] + red[0][1] + red[0][2] + red[0][3];
   sumsq = red[1][0] + red[1][1] + red[1][2] + red[1][3];
   const float mean = sum / (float)n;
-  const float var = sumsq / (float)n - mean * mean;
+  const float var = fmaxf(sumsq / (float)n - mean * mean, 0.f);  // cancellation on a near-constant row must not go negative
   const float rstd = 1.0f / sqrtf(var + eps);
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {

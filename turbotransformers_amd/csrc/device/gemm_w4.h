@@ -106,17 +106,44 @@ __device__ __forceinline__ void pair_swap(S& a, S& b) {
 #endif
 }
 
+// One accumulator register into an ordinary one, here and now: without it the compiler copies every accumulator of a
+// tile out of the AGPR half at the end of the K loop, 192 or 256 live registers at once.
+template <typename S>
+__device__ __forceinline__ S acc_read(S v) {
+  S r;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(v));
+  return r;
+}
+
+// 16 bytes into the wavefront's own epilogue strip.  Written as an instruction rather than as a C++ store: with
+// global->LDS DMA loads in flight (the next tile's first K steps) the compiler guards every LDS store it knows of
+// with a wait for ALL outstanding vector memory operations, i.e. also for the global stores of the previous row
+// block, one HBM round trip per block.  The strip is disjoint from the DMA stages, and LDS operations of one
+// wavefront complete in order, so the reads that follow need no more than their usual counter wait.
+__device__ __forceinline__ void strip_write(uint32_t lds_addr, const Chunk& x) {
+  asm volatile("ds_write_b128 %0, %1" : : "v"(lds_addr), "v"(__builtin_bit_cast(Quad, x)) : "memory");
+}
+
 // Bias of eight consecutive columns, kept in storage precision (16 bytes for 2-byte types) until it is added.
 template <typename BT>
 struct BiasVec {
   static constexpr int kPer = 16 / sizeof(BT), kChunksPerVec = 8 / kPer;
   Chunk raw[kChunksPerVec];
   bool present;
-  __device__ __forceinline__ void load(const BT* bias, int ncol) {
+  // `fallback`: any readable, 16-byte aligned address with 32 bytes behind it.  Without a bias the loads go there
+  // (and are ignored): a load under a branch would be waited for at the end of its block, one round trip each.
+  __device__ __forceinline__ void load(const BT* bias, int ncol, const void* fallback) {
     present = bias != nullptr;
-    if (present) {
+    const BT* src = present ? bias + ncol : static_cast<const BT*>(fallback);
 #pragma unroll
-      for (int c = 0; c < kChunksPerVec; ++c) raw[c] = *reinterpret_cast<const Chunk*>(bias + ncol + c * kPer);
+    for (int c = 0; c < kChunksPerVec; ++c) raw[c] = *reinterpret_cast<const Chunk*>(src + c * kPer);
+  }
+  __device__ __forceinline__ void widen(float (&out)[8]) const {
+#pragma unroll
+    for (int c = 0; c < kChunksPerVec; ++c) {
+      const Vec<BT, kPer> v = __builtin_bit_cast(Vec<BT, kPer>, raw[c]);
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) out[c * kPer + e] = to_float(v.v[e]);
     }
   }
   template <typename S>
@@ -133,6 +160,35 @@ struct BiasVec {
 
 constexpr int kW4Threads = 256;
 
+// Epilogues whose output is one row-major matrix: base address and leading dimension, so that the kernel can
+// store through a buffer resource (32-bit offsets, rows past M dropped by the hardware's range check).
+template <typename Epi>
+struct LinearDest : std::false_type {
+  static __device__ __forceinline__ void* base(const Epi&) { return nullptr; }
+  static __device__ __forceinline__ int64_t ldc(const Epi&) { return 0; }
+};
+template <typename T, int ACT, bool HAS_ACT>
+struct LinearDest<EpiBias<T, ACT, HAS_ACT, false>> : std::true_type {
+  static __device__ __forceinline__ void* base(const EpiBias<T, ACT, HAS_ACT, false>& e) { return e.c; }
+  static __device__ __forceinline__ int64_t ldc(const EpiBias<T, ACT, HAS_ACT, false>& e) { return e.ldc; }
+};
+template <typename T>
+struct LinearDest<EpiAlphaBeta<T>> : std::true_type {
+  static __device__ __forceinline__ void* base(const EpiAlphaBeta<T>& e) { return e.c; }
+  static __device__ __forceinline__ int64_t ldc(const EpiAlphaBeta<T>& e) { return e.ldc; }
+};
+
+#ifdef TTMI_W4_TRACE
+__device__ unsigned long long w4_trace[4][16][8][2];
+#define W4_STAMP(slot)                                                                    \
+  if (blockIdx.x == TTMI_W4_TRACE && lane == 0 && t < 16) {                               \
+    w4_trace[wave][t][slot][0] = __builtin_readcyclecounter();                            \
+    w4_trace[wave][t][slot][1] = wall_clock64();                                          \
+  }
+#else
+#define W4_STAMP(slot)
+#endif
+
 // LDS of the kernel: two K-loop stages plus one private epilogue strip per wavefront (MF rows x BN/2 columns of
 // the 2-byte output type; rows padded by 16 bytes when that does not fit a power-of-two swizzle).
 template <int BN, int MF>
@@ -145,6 +201,7 @@ constexpr int w4_lds_bytes() { return 2 * (256 + BN) * kRowBytes + 4 * MF * w4_s
 template <typename T, int BN, int MF, typename Epi>
 __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, const Epi epi) {
   static_assert(sizeof(T) == 2, "16-bit operands");
+  static_assert(MF == 32, "the epilogue pairs lanes l and l + 32");
   constexpr int BM = 256;
   constexpr int BK = kRowBytes / sizeof(T);
   constexpr int RB = 128 / MF, CB = BN / 2 / MF;   // blocks per wavefront: rows, columns
@@ -226,8 +283,16 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, bs + (i - A_LOADS) * 1024, 16, vob[i - A_LOADS], b_soff + dma_k * kRowBytes, 0, 0);
     }
   };
+  // the output matrix of a linear epilogue: rows at and past M lie outside the resource and their stores are dropped
+  const uint32_t ldc_bytes = (uint32_t)LinearDest<Epi>::ldc(epi) * (uint32_t)sizeof(T);
+  const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(LinearDest<Epi>::base(epi), 0, (int)min((int64_t)g.m * ldc_bytes, (int64_t)0x7fffffff), 0x00020000);
+  auto store_c = [&](const Chunk& x, uint32_t voff, uint32_t soff) __attribute__((always_inline)) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(Quad, x), rsrc_c, (int)voff, (int)soff, 0);
+  };
 #else
   auto dma_issue_one = [&](int) {};
+  const uint32_t ldc_bytes = 0;
+  auto store_c = [&](const Chunk&, uint32_t, uint32_t) {};
 #endif
   auto dma_issue = [&](auto lo_tag, auto hi_tag) __attribute__((always_inline)) {
     constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
@@ -319,6 +384,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   read_frags(0, 0, fa[0], fb[0]);
 
   char* strip = smem + 2 * STAGE + wave * (MF * PITCH);
+  const uint32_t strip_lds = (uint32_t)reinterpret_cast<uintptr_t>(strip);  // low half of a generic LDS address = LDS offset
   int tile = first;
   for (int t = 0; t < my_tiles; ++t, tile += stride) {
     int tile_m, tile_n;
@@ -326,6 +392,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     bool swap = true;
     if constexpr (HasColumnPass<Epi>::value) swap = !(epi.column_pass() && n0 >= epi.first_column_of_pass());
+    W4_STAMP(0)
 
 #pragma unroll
     for (int i = 0; i < RB; ++i)
@@ -337,73 +404,110 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     const auto* bias = epi.bias_ptr();
     using BiasT = typename std::remove_cv<typename std::remove_pointer<decltype(bias)>::type>::type;
     const int m_lim = g.m, n_lim = g.n;
+    // bias of this lane's column groups, requested now so that it has landed when the epilogue wants it
+    constexpr int NV = CB * 2;
+    BiasVec<BiasT> bv[NV];
     if (swap) {
+#pragma unroll
+      for (int v = 0; v < NV; ++v) bv[v].load(bias, min(n0 + wn0 + ((v / 2) * 4 + (v % 2) * 2 + lgrp) * 8, n_lim - 8), g.b);  // N % 8 == 0
+    }
+    W4_STAMP(1)
+    if (swap) {
+#ifdef TTMI_W4_TRACE
+      k_step(std::integral_constant<int, 0>{}, std::true_type{});
+      W4_STAMP(4)
+      k_step(std::integral_constant<int, 1>{}, std::true_type{});
+      W4_STAMP(5)
+      for (int kt = 2; kt < ksteps; kt += 2) {
+#else
       for (int kt = 0; kt < ksteps; kt += 2) {
+#endif
         k_step(std::integral_constant<int, 0>{}, std::true_type{});
         k_step(std::integral_constant<int, 1>{}, std::true_type{});
       }
-      // A lane now owns, per block (pair), eight consecutive columns of one row: + bias, finish(), round to T,
-      // 16 bytes into the wavefront's strip; the strip goes out row-contiguous, 16 bytes per lane.
-      constexpr int NV = MF == 32 ? CB * 2 : CB / 2;
-      BiasVec<BiasT> bv[NV];
-      int chunk_of[NV];
+      W4_STAMP(2)
+      // A lane now owns, per block, runs of four consecutive columns of one row; a pair swap makes them runs of
+      // eight: + bias, finish(), round to T, 16 bytes into the wavefront's strip, which leaves row-contiguous, 16
+      // bytes per lane.  A lone wavefront on a SIMD hides no latency by itself, so the order is written out: the
+      // arithmetic of row block i runs while the strip reads of block i-1 are in flight, then the stores of block
+      // i-1 go out back to back, then block i is written to the strip and its reads are issued.
+      constexpr int PASSES = MF * CPR / kWave;
+      static_assert(MF * CPR % kWave == 0, "whole passes over a strip");
+      int rd_off[PASSES], st_row[PASSES], st_col[PASSES], wr_off[NV];
 #pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        if constexpr (MF == 32) chunk_of[v] = (v / 2) * 4 + (v % 2) * 2 + lgrp;
-        else chunk_of[v] = 2 * (2 * v + (lgrp & 1)) + (lgrp >> 1);
-        bv[v].load(bias, min(n0 + wn0 + chunk_of[v] * 8, n_lim - 8));  // N % 8 == 0
+      for (int pass = 0; pass < PASSES; ++pass) {
+        const int idx = pass * kWave + lane;
+        const int r = idx / CPR, c = idx % CPR;
+        rd_off[pass] = r * PITCH + ((XOR_STRIP ? (c ^ (r & (CPR - 1))) : c) << 4);
+        st_row[pass] = r;
+        st_col[pass] = c * 8;
       }
 #pragma unroll
-      for (int i = 0; i < RB; ++i) {
+      for (int v = 0; v < NV; ++v) {
+        const int c = (v / 2) * 4 + (v % 2) * 2 + lgrp;
+        wr_off[v] = lrow * PITCH + ((XOR_STRIP ? (c ^ (lrow & (CPR - 1))) : c) << 4);
+      }
+      float bf[NV][8];
+      const bool has_bias = bias != nullptr;  // uniform
+      if (has_bias) {
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-          float out[8];
-          if constexpr (MF == 32) {
+        for (int v = 0; v < NV; ++v) bv[v].widen(bf[v]);
+      }
+      const bool whole_width = n0 + BN <= n_lim;  // uniform
+      Chunk landed[PASSES];
+#pragma unroll
+      for (int i = 0; i <= RB; ++i) {
+        Chunk packed[NV];
+        if (i < RB) {
+#pragma unroll
+          for (int v = 0; v < NV; ++v) {
             const int j = v / 2, gp = v % 2;
+            float out[8];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              float a = acc[i][j][8 * gp + e], b = acc[i][j][8 * gp + 4 + e];
+              float a = acc_read(acc[i][j][8 * gp + e]), b = acc_read(acc[i][j][8 * gp + 4 + e]);
               pair_swap<32>(a, b);
               out[e] = a;
               out[4 + e] = b;
             }
+            if (has_bias) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) out[e] += bf[v][e];
+            }
+            T rounded[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) rounded[e] = from_float<T>(epi.finish(out[e]));
+            packed[v] = pack_chunk(rounded);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (i > 0) {
+          const int row0 = m0 + wm0 + (i - 1) * MF;
+          if constexpr (LinearDest<Epi>::value) {
+            const uint32_t soff = (uint32_t)row0 * ldc_bytes + (uint32_t)(n0 + wn0) * (uint32_t)sizeof(T);
+#pragma unroll
+            for (int pass = 0; pass < PASSES; ++pass)
+              if (whole_width || n0 + wn0 + st_col[pass] < n_lim)
+                store_c(landed[pass], (uint32_t)st_row[pass] * ldc_bytes + (uint32_t)st_col[pass] * (uint32_t)sizeof(T), soff);
           } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              float a = acc[i][2 * v][e], b = acc[i][2 * v + 1][e];
-              pair_swap<16>(a, b);
-              out[e] = a;
-              out[4 + e] = b;
+            for (int pass = 0; pass < PASSES; ++pass) {
+              const int m = row0 + st_row[pass], ncol = n0 + wn0 + st_col[pass];
+              if (m < m_lim && ncol < n_lim) *reinterpret_cast<Chunk*>(epi.dest8(m, ncol)) = landed[pass];
             }
           }
-          {
-            // the bias stays packed between uses: widened once per strip it would occupy 64 registers across the
-            // whole epilogue (the asm statement keeps the compiler from hoisting the conversion out of the strip loop)
-            BiasVec<BiasT> b = bv[v];
-            asm volatile("" : "+v"(b.raw[0].w[0]), "+v"(b.raw[0].w[1]), "+v"(b.raw[0].w[2]), "+v"(b.raw[0].w[3]));
-            b.add_to(out);
-          }
-          T packed[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) packed[e] = from_float<T>(epi.finish(out[e]));
-          const int pc = XOR_STRIP ? (chunk_of[v] ^ (lrow & (CPR - 1))) : chunk_of[v];
-          *reinterpret_cast<Chunk*>(strip + lrow * PITCH + (pc << 4)) = pack_chunk(packed);
-          __builtin_amdgcn_sched_barrier(0);  // one group of eight at a time: no wholesale hoisting of accumulator reads
         }
-        // same wavefront, LDS operations complete in order: no barrier between the writes and the reads
-        constexpr int PASSES = (MF * CPR + kWave - 1) / kWave;
+        __builtin_amdgcn_sched_barrier(0);
+        if (i < RB) {
+          // same wavefront, LDS operations complete in order: no barrier between the writes and the reads
 #pragma unroll
-        for (int pass = 0; pass < PASSES; ++pass) {
-          const int idx = pass * kWave + lane;
-          const int r = idx / CPR, c = idx % CPR;
-          if (MF * CPR % kWave != 0 && r >= MF) continue;
-          const int pc = XOR_STRIP ? (c ^ (r & (CPR - 1))) : c;
-          const Chunk x = *reinterpret_cast<const Chunk*>(strip + r * PITCH + (pc << 4));
-          const int m = m0 + wm0 + i * MF + r, ncol = n0 + wn0 + c * 8;
-          if (m < m_lim && ncol < n_lim) *reinterpret_cast<Chunk*>(epi.dest8(m, ncol)) = x;
+          for (int v = 0; v < NV; ++v) strip_write(strip_lds + (uint32_t)wr_off[v], packed[v]);
+#pragma unroll
+          for (int pass = 0; pass < PASSES; ++pass) landed[pass] = *reinterpret_cast<const Chunk*>(strip + rd_off[pass]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
+      W4_STAMP(3)
     } else {
       if constexpr (HasColumnPass<Epi>::value) {
         for (int kt = 0; kt < ksteps; kt += 2) {
@@ -464,6 +568,11 @@ static bool w4_eligible(const GemmArgs& g, int batch, bool aligned) {
   const int64_t limit = (int64_t)1 << 31;
   return (int64_t)g.m * g.lda * (int64_t)sizeof(T) < limit && (int64_t)g.n * g.ldb * (int64_t)sizeof(T) < limit;
 }
+// The output of a linear epilogue is addressed with 32-bit offsets as well.
+template <typename T>
+static bool w4_output_fits(const GemmArgs& g, int64_t ldc) {
+  return (int64_t)g.m * ldc * (int64_t)sizeof(T) < ((int64_t)1 << 31);
+}
 
 template <typename T, int BN, typename Epi>
 static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s) {
@@ -512,7 +621,7 @@ struct LargeTileKernel<T, EpiBias<T, ACT, HAS_ACT, false>, typename std::enable_
       const char* force = std::getenv("TTMI_LARGE_TILE");
       if (force == nullptr || force[0] != '1') return false;
     }
-    return w4_wanted<T>(g, epi, batch, aligned);
+    return w4_output_fits<T>(g, epi.ldc) && w4_wanted<T>(g, epi, batch, aligned);
   }
   static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
 };
@@ -520,7 +629,7 @@ template <typename T>
 struct LargeTileKernel<T, EpiAlphaBeta<T>, typename std::enable_if<sizeof(T) == 2>::type> {
   using Epi = EpiAlphaBeta<T>;
   static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
-    return epi.beta == 0.f && w4_wanted<T>(g, epi, batch, aligned);
+    return epi.beta == 0.f && w4_output_fits<T>(g, epi.ldc) && w4_wanted<T>(g, epi, batch, aligned);
   }
   static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
 };

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
   sum = group_sum<G>(sum);
   sumsq = group_sum<G>(sumsq);
   const float mean = sum / (float)n;
-  const float var = sumsq / (float)n - mean * mean;
+  const float var = fmaxf(sumsq / (float)n - mean * mean, 0.f);  // cancellation on a near-constant row must not go negative
   const float rstd = 1.0f / sqrtf(var + eps);
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kBlock) void layer_norm_block(T* __restrict__ out, 
     sumsq += red[1][w];
   }
   const float mean = sum / (float)n;
-  const float var = sumsq / (float)n - mean * mean;
+  const float var = fmaxf(sumsq / (float)n - mean * mean, 0.f);  // cancellation on a near-constant row must not go negative
   const float rstd = 1.0f / sqrtf(var + eps);
   for (int c = threadIdx.x; c < n; c += kBlock) {
     float x = to_float(orow[c]);

@@ -14,6 +14,12 @@ DeviceContext& DeviceContext::GetInstance() {
   return ctx;
 }
 
+void DeviceContext::set_stream(void* s) {
+  if (s == stream_) return;
+  TT_DEVICE_CALL(ttmi_stream_sync(stream_));
+  stream_ = s;
+}
+
 void DeviceContext::Wait() const {
   TT_DEVICE_CALL(ttmi_stream_sync(stream_));
   TT_DEVICE_CALL(ttmi_check_async());
@@ -35,14 +41,19 @@ DeviceContext::SeqPlan DeviceContext::GetSeqPlan(const std::vector<int64_t>& len
   const int64_t total = std::accumulate(lens.begin(), lens.end(), (int64_t)0);
   const int64_t max_seq = *std::max_element(lens.begin(), lens.end());
   if (!(lens == plan_lens_ && plan_stream_ == stream_)) {
+    // The device tables are rewritten in stream order, behind the kernels that still read the previous batch's.
     if (batch + 1 > plan_cu_cap_) {
-      // Retired buffers may still be read by kernels in flight: drain the stream first.
+      // Retired buffers may still be read by kernels in flight: drain the stream first (growth is rare).
       TT_DEVICE_CALL(ttmi_stream_sync(stream_));
       if (plan_cu_) TT_DEVICE_CALL(ttmi_free(plan_cu_));
-      if (plan_staging_) TT_DEVICE_CALL(ttmi_host_free(plan_staging_));
       plan_cu_cap_ = std::max<int64_t>(64, 2 * (batch + 1));
       TT_DEVICE_CALL(ttmi_malloc(reinterpret_cast<void**>(&plan_cu_), plan_cu_cap_ * sizeof(int32_t)));
-      TT_DEVICE_CALL(ttmi_host_malloc(reinterpret_cast<void**>(&plan_staging_), plan_cu_cap_ * sizeof(int32_t)));
+      for (StagingSlot& slot : plan_slots_) {
+        if (slot.words) TT_DEVICE_CALL(ttmi_host_free(slot.words));
+        TT_DEVICE_CALL(ttmi_host_malloc(reinterpret_cast<void**>(&slot.words), plan_cu_cap_ * sizeof(int32_t)));
+        if (slot.copied == nullptr) TT_DEVICE_CALL(ttmi_event_create(&slot.copied));
+        slot.in_use = false;
+      }
     }
     if (total > plan_rows_cap_) {
       TT_DEVICE_CALL(ttmi_stream_sync(stream_));
@@ -50,9 +61,13 @@ DeviceContext::SeqPlan DeviceContext::GetSeqPlan(const std::vector<int64_t>& len
       plan_rows_cap_ = std::max<int64_t>(4096, 2 * total);
       TT_DEVICE_CALL(ttmi_malloc(reinterpret_cast<void**>(&plan_rows_), plan_rows_cap_ * sizeof(int32_t)));
     }
-    // The pinned staging words are read by the async copy: the previous upload must be done.
-    TT_DEVICE_CALL(ttmi_stream_sync(stream_));
-    TT_DEVICE_CALL(ttmi_build_cu_seqlens(lens.data(), batch, plan_staging_, plan_cu_, stream_));
+    StagingSlot& slot = plan_slots_[plan_next_slot_];
+    plan_next_slot_ = (plan_next_slot_ + 1) % kPlanSlots;
+    // the pinned words are read by an asynchronous copy: the one that used this slot last must be done
+    if (slot.in_use) TT_DEVICE_CALL(ttmi_event_sync(slot.copied));
+    TT_DEVICE_CALL(ttmi_build_cu_seqlens(lens.data(), batch, slot.words, plan_cu_, stream_));
+    TT_DEVICE_CALL(ttmi_event_record(slot.copied, stream_));
+    slot.in_use = true;
     if (total > 0) TT_DEVICE_CALL(ttmi_build_token_rows(plan_cu_, batch, max_seq, total, plan_rows_, stream_));
     plan_lens_ = lens;
     plan_stream_ = stream_;

@@ -20,7 +20,9 @@ class DeviceContext {
   static DeviceContext& GetInstance();
 
   void* stream() const { return stream_; }
-  void set_stream(void* s) { stream_ = s; }
+  // Switching to another stream first drains the old one: cached state (packed weights, recycled allocator blocks,
+  // the batch tables below) was produced by work on the old stream and carries no other dependency.
+  void set_stream(void* s);
   void Wait() const;  // synchronise the stream and surface asynchronous kernel errors
 
   int compute_units();
@@ -43,7 +45,16 @@ class DeviceContext {
   std::vector<int64_t> plan_lens_;
   int32_t* plan_cu_ = nullptr;
   int32_t* plan_rows_ = nullptr;
-  int32_t* plan_staging_ = nullptr;
+  // Pinned staging words of the cu_seqlens upload: a small ring, each slot with the event recorded behind its copy, so
+  // that a new list of lengths waits only for the copy that used its slot four uploads ago, never for the stream.
+  static constexpr int kPlanSlots = 4;
+  struct StagingSlot {
+    int32_t* words = nullptr;
+    void* copied = nullptr;  // event
+    bool in_use = false;
+  };
+  StagingSlot plan_slots_[kPlanSlots];
+  int plan_next_slot_ = 0;
   int64_t plan_cu_cap_ = 0, plan_rows_cap_ = 0;
   void* plan_stream_ = nullptr;
 };

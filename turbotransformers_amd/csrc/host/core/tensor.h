@@ -80,6 +80,8 @@ class Tensor {
   const Tensor* shadow() const { return shadow_.get(); }
   Tensor* EnsureShadow();
   void DropShadow() { shadow_.reset(); }
+  // Hand the fp32 copy to the caller (null when there is none); the tensor keeps its own buffer.
+  std::unique_ptr<Tensor> TakeShadow() { return std::move(shadow_); }
 
   bool is_null() const { return managed_ == nullptr && !is_view_; }
 

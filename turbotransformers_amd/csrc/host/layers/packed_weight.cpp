@@ -11,6 +11,7 @@ const void* PackedWeight::Get(const core::Tensor& w, bool is_trans_weight) const
   TT_ENFORCE_EQ(w.n_dim(), (size_t)2, "weights must be 2-D");
   kernels::RequireGpu(w, "weight");
   if (is_trans_weight) return w.raw();
+  std::lock_guard<std::mutex> lock(mutex_);
   if (source_ != w.raw() || packed_.is_null()) {
     const int64_t K = w.shape(0), N = w.shape(1);
     packed_.ReshapeAs(w.dtype(), {N, K}, w.device_type(), w.device_id(), "PackedWeight");

@@ -4,6 +4,8 @@
 // afterwards only returns the pointer.
 #pragma once
 
+#include <mutex>
+
 #include "core/tensor.h"
 
 namespace turbo_transformers {
@@ -18,6 +20,7 @@ class PackedWeight {
   static int64_t InDim(const core::Tensor& w, bool is_trans_weight) { return is_trans_weight ? w.shape(1) : w.shape(0); }
 
  private:
+  mutable std::mutex mutex_;  // two threads may make the first call of one layer object together
   mutable core::Tensor packed_;
   mutable const void* source_ = nullptr;
 };

@@ -24,6 +24,7 @@ QuantizedLinear::QuantizedLinear(core::Tensor weight, core::Tensor bias, const s
 }
 
 void QuantizedLinear::Prepare() const {
+  std::lock_guard<std::mutex> lock(prepare_mutex_);
   if (prepared_) return;
   kernels::RequireGpu(weight_, "QuantizedLinear");
   TT_ENFORCE_EQ(weight_.n_dim(), (size_t)2, "weight must be [in, out]");

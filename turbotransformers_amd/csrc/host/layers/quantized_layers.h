@@ -42,6 +42,7 @@ class QuantizedLinear {
   int act_ = -1;  // ttmi_act; -1 = none
   mutable core::Tensor q_weight_, w_scales_, q_input_, act_scale_;
   mutable bool prepared_ = false;
+  mutable std::mutex prepare_mutex_;  // the one-time weight quantisation; calls on one object are otherwise not concurrent
 };
 
 class QuantizedBertAttention {

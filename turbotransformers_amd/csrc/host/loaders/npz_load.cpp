@@ -102,40 +102,58 @@ NpyArray ParseNpy(Reader& file, uint64_t size) {
     header_len = Get<uint32_t>(head + 8);
     consumed = 12;
   }
+  TT_ENFORCE(consumed + header_len <= size, "npy header is longer than its member");
   std::string header(header_len, '\0');
   file.Read(&header[0], header_len);
   consumed += header_len;
 
   NpyArray arr;
+  // Every position found in the header text is checked: a malformed member must end in EnforceNotMet, not in
+  // std::out_of_range from substr or std::invalid_argument from stoi.
+  auto need = [&](size_t pos, const char* what) -> size_t {
+    TT_ENFORCE(pos != std::string::npos && pos < header.size(), "malformed npy header (%s)", what);
+    return pos;
+  };
   auto find_value = [&](const std::string& key) -> size_t {
     const size_t k = header.find("'" + key + "'");
     TT_ENFORCE(k != std::string::npos, "npy header lacks %s", key.c_str());
-    return header.find(':', k) + 1;
+    return need(header.find(':', k), key.c_str()) + 1;
   };
   size_t p = find_value("descr");
-  p = header.find('\'', p);
-  const std::string descr = header.substr(p + 1, header.find('\'', p + 1) - p - 1);
-  TT_ENFORCE(descr.size() >= 3 && (descr[0] == '<' || descr[0] == '|'), "unsupported npy dtype %s", descr.c_str());
+  p = need(header.find('\'', p), "descr");
+  const size_t descr_end = need(header.find('\'', p + 1), "descr");
+  const std::string descr = header.substr(p + 1, descr_end - p - 1);
+  TT_ENFORCE(descr.size() >= 3 && descr.size() <= 4 && (descr[0] == '<' || descr[0] == '|') &&
+                 descr.find_first_not_of("0123456789", 2) == std::string::npos,
+             "unsupported npy dtype %s", descr.c_str());
   arr.kind = descr[1];
   arr.word_size = std::stoi(descr.substr(2));
   TT_ENFORCE((arr.kind == 'f' && (arr.word_size == 4 || arr.word_size == 2)) || (arr.kind == 'i' && arr.word_size == 8),
              "unsupported npy dtype %s (float32, float16 and int64 are read)", descr.c_str());
   p = find_value("fortran_order");
-  TT_ENFORCE(header.compare(header.find_first_not_of(' ', p), 5, "False") == 0, "fortran-ordered arrays are not supported");
+  p = need(header.find_first_not_of(' ', p), "fortran_order");
+  TT_ENFORCE(header.compare(p, 5, "False") == 0, "fortran-ordered arrays are not supported");
   p = find_value("shape");
-  const size_t lp = header.find('(', p), rp = header.find(')', lp);
+  const size_t lp = need(header.find('(', p), "shape");
+  const size_t rp = need(header.find(')', lp), "shape");
   std::string dims = header.substr(lp + 1, rp - lp - 1);
   size_t q = 0;
+  uint64_t numel = 1;
   while (q < dims.size()) {
     while (q < dims.size() && (dims[q] == ' ' || dims[q] == ',')) ++q;
     if (q >= dims.size()) break;
     size_t e = q;
     while (e < dims.size() && dims[e] >= '0' && dims[e] <= '9') ++e;
-    TT_ENFORCE(e > q, "malformed npy shape");
-    arr.shape.push_back(std::stoll(dims.substr(q, e - q)));
+    TT_ENFORCE(e > q && e - q <= 18, "malformed npy shape");
+    const uint64_t dim = std::stoull(dims.substr(q, e - q));
+    // the product is bounded by the member's size at every step, so it cannot wrap around
+    TT_ENFORCE(dim == 0 || numel <= size / dim, "npy shape is larger than its member");
+    numel *= dim;
+    arr.shape.push_back((int64_t)dim);
     q = e;
   }
-  const uint64_t payload = (uint64_t)arr.numel() * arr.word_size;
+  TT_ENFORCE(numel <= size / (uint64_t)arr.word_size, "npy shape is larger than its member");
+  const uint64_t payload = numel * (uint64_t)arr.word_size;
   TT_ENFORCE_EQ(consumed + payload, size, "npy member size does not match its shape");
   arr.bytes.resize(payload);
   if (payload) file.Read(arr.bytes.data(), payload);
@@ -186,6 +204,11 @@ std::map<std::string, NpyArray> LoadNpz(const std::string& filename) {
     std::vector<unsigned char> extra(extra_len);
     if (extra_len) file.Read(extra.data(), extra_len);
     ApplyZip64(extra.data(), extra_len, &usize, &csize, &local);
+    // sizes come from the file: bound them by it before anything is allocated from them (a deflated member expands
+    // by at most 1032:1)
+    TT_ENFORCE(csize <= (uint64_t)file_size && local <= (uint64_t)file_size && usize / 1032 <= (uint64_t)file_size,
+               "%s: member %s has sizes beyond the file", filename.c_str(), name.c_str());
+    TT_ENFORCE(method != 0 || usize <= (uint64_t)file_size, "%s: member %s is larger than the file", filename.c_str(), name.c_str());
     pos += 46 + name_len + extra_len + comment_len;
     // numpy.savez stores members (method 0); numpy.savez_compressed, which the reference's converter
     // uses (tools/convert_huggingface_bert_pytorch_to_npz.py:71), deflates them (method 8)

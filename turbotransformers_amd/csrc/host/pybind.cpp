@@ -103,6 +103,9 @@ PYBIND11_MODULE(turbo_transformers_cxx, m) {
              auto* dlpack = tensor.ToDLPack();
              return py::capsule(dlpack, "dltensor", DLPackCapsuleDestructor);
            })
+      // The unrounded fp32 values a bfloat16 LayerNorm output travels with (None when there are none): the final
+      // hidden state of a bfloat16 model before its rounding to 8 mantissa bits.  No counterpart in the reference.
+      .def("take_fp32_shadow", [](Tensor& tensor) -> std::unique_ptr<Tensor> { return tensor.TakeShadow(); })
       .def("n_dim", &Tensor::n_dim)
       .def("shape", [](const Tensor& t, int pos) { return t.shape(pos); })
       .def("float_data", [](const Tensor& t) { return reinterpret_cast<uintptr_t>(t.data<float>()); })

@@ -296,7 +296,9 @@ class BertModel:
                  head_mask: Optional[AnyTensor] = None, inputs_embeds: Optional[AnyTensor] = None,
                  output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
                  pooling_type: PoolingType = PoolingType.FIRST, pooler_output: Optional[AnyTensor] = None,
-                 return_type: Optional[ReturnType] = None):
+                 return_type: Optional[ReturnType] = None, output_fp32_hidden_state: bool = False):
+        """output_fp32_hidden_state (not in the reference): bfloat16 models keep their residual stream in fp32; True
+        appends that unrounded final hidden state (a float32 torch tensor, or None for other dtypes) to the result."""
         encoder_outputs = self.bertmodel_nopooler(inputs, attention_masks, token_type_ids, position_ids,
                                                   inputs_embeds=inputs_embeds, output_attentions=output_attentions,
                                                   output_hidden_states=output_hidden_states,
@@ -306,7 +308,11 @@ class BertModel:
         self.seq_pool = SequencePool(PoolingMap[pooling_type])
         pooled = self.seq_pool(input_tensor=sequence_output, return_type=ReturnType.turbo_transformers)
         pooler_output = self.pooler(pooled, return_type, pooler_output)
-        return (convert_returns_as_type(sequence_output, return_type), pooler_output) + encoder_outputs[1:]
+        extra = ()
+        if output_fp32_hidden_state:
+            shadow = sequence_output.take_fp32_shadow()
+            extra = (convert_returns_as_type(shadow, ReturnType.TORCH) if shadow is not None else None, )
+        return (convert_returns_as_type(sequence_output, return_type), pooler_output) + encoder_outputs[1:] + extra
 
     @staticmethod
     def from_torch(model, device: Optional[torch.device] = None, backend: Optional[str] = None, use_memory_opt=False):

@@ -17,7 +17,10 @@ class ReturnType(enum.Enum):
 
 def convert_returns_as_type(tensor, rtype: Optional[ReturnType]):
     """cxx.Tensor -> cxx.Tensor | torch.Tensor | numpy.  TORCH hands the buffer over through
-    DLPack without a copy: the cxx.Tensor is empty afterwards and torch owns the memory."""
+    DLPack without a copy: the cxx.Tensor is empty afterwards and torch owns the memory; nothing waits for the
+    device, so an error a kernel reported (an embedding id out of range, whose row is NaN in the result) is raised
+    by the next `cxx.synchronize()`.  NUMPY copies to the host, which waits for the device anyway, and raises
+    such an error itself."""
     if rtype is None:
         rtype = ReturnType.TORCH
     if rtype == ReturnType.turbo_transformers:
@@ -26,5 +29,7 @@ def convert_returns_as_type(tensor, rtype: Optional[ReturnType]):
         return dlpack.from_dlpack(tensor.to_dlpack())
     if rtype == ReturnType.NUMPY:
         t = dlpack.from_dlpack(tensor.to_dlpack())
-        return t.float().cpu().numpy()
+        host = t.float().cpu().numpy()
+        cxx.synchronize()
+        return host
     raise NotImplementedError()

@@ -323,6 +323,16 @@ TTMI_API int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, i
                              int64_t lda, int64_t ldb, int64_t ldc, int epilogue,
                              const ttmi_epilogue_args* args, int dtype, void* stream);
 
+/* Which kernel variant ttmi_gemm (epilogue TTMI_EPI_NONE, args NULL) or ttmi_gemm_fused would launch for an
+ * aligned, densely packed product of this shape, as text: family (reg = register-staged, dma = global->LDS DMA,
+ * dma_agpr = DMA with accumulators in AGPRs), wavefronts per workgroup, tile, K split; e.g. "dma8w_256x256".
+ * Nothing is launched.  No counterpart in the reference (cuBLAS picks its kernels out of sight); measurement
+ * scripts use it to tie recorded per-kernel figures to the variant they were recorded on.  For the QKV epilogues
+ * `args` supplies seq / heads / head_dim / v_seq_pitch (and batch); pointers in it are ignored. */
+TTMI_API int ttmi_gemm_describe(int64_t m, int64_t n, int64_t k, int epilogue, const ttmi_epilogue_args* args, int dtype,
+                                char* out, size_t capacity);
+
+
 /* int8 path (quantized BERT: int8 x int8 -> int32 accumulators, exact).
  * ttmi_quantize_rows_i8: per-tensor symmetric dynamic scale from max|x| over the whole
  *   [m,k] activation: scale = max|x|/127 (1 if the tensor is all zero), q = clamp(rint(x/scale), -127, 127).

@@ -222,3 +222,19 @@ def test_npz_reader_refuses_sizes_beyond_the_file(tmp_path):
     open(path, "wb").write(bytes(data))
     with pytest.raises(RuntimeError):
         cxx.load_npz(path)
+
+
+def test_gemm_describe_names_the_variant_without_a_device():
+    """ttmi_gemm_describe runs the launchers' own selection with launching switched off, so it answers on a machine
+    without a GPU: a family, the wavefronts per workgroup, the tile and the K split."""
+    import ctypes
+    import re
+    lib = capi.load()
+    buf = ctypes.create_string_buffer(64)
+    args = capi.EpilogueArgs()
+    args.act = capi.ACT_GELU
+    for m, n, k, epi in [(32768, 3072, 768, capi.EPI_BIAS_ACT), (32768, 768, 3072, capi.EPI_NONE), (128, 768, 3072, capi.EPI_NONE),
+                         (2560, 768, 3072, capi.EPI_BIAS)]:
+        capi.check(lib.ttmi_gemm_describe(m, n, k, epi, ctypes.byref(args), capi.F16, buf, 64))
+        assert re.fullmatch(r"(reg|dma|dma_agpr)\d+w_\d+x\d+(_splitk\d+)?", buf.value.decode()), buf.value
+    assert lib.ttmi_gemm_describe(128, 768, 3072, capi.EPI_NONE, None, capi.F16, buf, 4) != 0  # too small for the answer

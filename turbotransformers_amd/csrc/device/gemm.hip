@@ -1,5 +1,7 @@
 // C ABI of the MFMA GEMM family: argument checks, epilogue selection and the static scratch buffer.
 // The kernels, epilogues and launch heuristics live in gemm_impl.h.
+#include <cstring>
+
 #include "gemm_impl.h"
 #include "gemm_w4.h"
 
@@ -193,6 +195,30 @@ int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n,
         return fail(TTMI_EINVAL, "unknown epilogue");
     }
   });
+  return 0;
+}
+
+int ttmi_gemm_describe(int64_t m, int64_t n, int64_t k, int epilogue, const ttmi_epilogue_args* args, int dtype, char* out,
+                       size_t capacity) {
+  TTMI_REQUIRE(out != nullptr && capacity > 0, "no room for the answer");
+  // operands that pass every alignment test; nothing dereferences them in a dry run
+  void* fake = reinterpret_cast<void*>((uintptr_t)1 << 20);
+  ttmi_epilogue_args filled{};
+  if (args != nullptr) filled = *args;
+  filled.bias = fake;
+  filled.residual = fake;
+  filled.q = filled.k = filled.v = fake;
+  if (epilogue == TTMI_EPI_QKV_SPLIT_PAD) filled.token_rows = static_cast<const int32_t*>(fake);
+  std::string name;
+  struct Install {
+    explicit Install(std::string* p) { tl_describe = p; }
+    ~Install() { tl_describe = nullptr; }
+  } install(&name);
+  const int rc = epilogue == TTMI_EPI_NONE ? ttmi_gemm(fake, fake, fake, m, n, k, k, k, n, 1, 1.f, 0.f, dtype, nullptr)
+                                           : ttmi_gemm_fused(fake, fake, fake, m, n, k, k, k, n, epilogue, &filled, dtype, nullptr);
+  if (rc != 0) return rc;
+  TTMI_REQUIRE(name.size() < capacity, "the answer does not fit");
+  std::memcpy(out, name.c_str(), name.size() + 1);
   return 0;
 }
 

@@ -26,6 +26,7 @@
 #include <map>
 #include <mutex>
 #include <set>
+#include <string>
 #include <type_traits>
 #include <utility>
 
@@ -1022,6 +1023,17 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
 }
 
 // ------------------------------------------------------------------------ launching -----
+// Dry run: while a thread has a string installed here, the launchers below write the name of the kernel variant
+// they would launch (tile, wavefronts, K split) into it and launch nothing.  ttmi_gemm_describe uses it, so the
+// answer comes from the very code path that picks the kernel.
+static thread_local std::string* tl_describe = nullptr;
+static bool describe_only(const char* family, int waves, int bm, int bn, int splits = 1) {
+  if (tl_describe == nullptr) return false;
+  *tl_describe = std::string(family) + std::to_string(waves) + "w_" + std::to_string(bm) + "x" + std::to_string(bn);
+  if (splits > 1) *tl_describe += "_splitk" + std::to_string(splits);
+  return true;
+}
+
 // Kernels that use more than 64 KB of dynamic LDS need the limit raised once per kernel and device.
 static int allow_large_lds(const void* kern, int bytes) {
   static std::mutex mu;
@@ -1039,6 +1051,7 @@ template <typename T, int BM, int BN, int WM, int WN, bool B_KN, bool ALIGNED, t
 static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   constexpr int NT = WM * WN * kWave;
   constexpr int LDS = 2 * (BM + BN) * kRowBytes;
+  if (describe_only("reg", WM * WN, BM, BN)) return 0;
   g.tiles_m = (g.m + BM - 1) / BM;
   g.tiles_n = (g.n + BN - 1) / BN;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
@@ -1071,6 +1084,7 @@ static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   constexpr int NT = WM * WN * kWave;
   constexpr int LDS = fast_lds_bytes<BM, BN, WM, WN>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
+  if (describe_only("dma", WM * WN, BM, BN)) return 0;
   g.tiles_m = (g.m + BM - 1) / BM;
   g.tiles_n = (g.n + BN - 1) / BN;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
@@ -1150,6 +1164,7 @@ static int pick_splits(int64_t m, int64_t n, int64_t ksteps, int64_t batch) {
 // `reduce(ws, slices, vec, stream)` launches the kernel that sums the slices and applies the epilogue.
 template <typename T, typename Reduce>
 static int launch_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStream_t s, const Reduce& reduce) {
+  if (describe_only("reg", 4, 64, 64, splits)) return 0;
   const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
   float* ws = nullptr;
   {
@@ -1175,6 +1190,7 @@ static int launch_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStre
 // (M = 2560, N = 768, K = 3072: 120 tiles, 48 K steps each).
 template <typename T, typename Reduce>
 static int launch_fast_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStream_t s, const Reduce& reduce) {
+  if (describe_only("dma", 4, 128, 128, splits)) return 0;
   const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
   float* ws = nullptr;
   {

@@ -578,6 +578,7 @@ template <typename T, int BN, typename Epi>
 static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s) {
   constexpr int LDS = w4_lds_bytes<BN, 32>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
+  if (describe_only("dma_agpr", 4, 256, BN)) return 0;
   g.tiles_m = (g.m + 255) / 256;
   g.tiles_n = (g.n + BN - 1) / BN;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;

@@ -314,6 +314,35 @@ struct EpiQkvSplit {
     T* base = (w == 0) ? q : (w == 1 ? k : v);
     return base + (((int64_t)b * heads + head) * seq + s) * dim + i;
   }
+  // dest(b, s, n) = col_part(n) + row_part(m): the address splits into a part that depends on the column only and an
+  // element offset that depends on the row only, so a kernel that stores many rows of few columns (or the reverse)
+  // does each division once.
+  __device__ __forceinline__ T* col_part(uint32_t n) const {
+    const uint32_t w = div_hidden.div(n);
+    const uint32_t rem = n - w * hidden;
+    const uint32_t head = div_dim.div(rem);
+    T* base = (w == 0) ? q : (w == 1 ? k : v);
+    return base + (int64_t)head * seq * dim + (rem - head * dim);
+  }
+  __device__ __forceinline__ int64_t row_part(int m) const {
+    const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;
+    const uint32_t b = div_seq.div(prow);
+    return ((int64_t)b * heads * seq + (prow - b * seq)) * dim;
+  }
+  // Whether `rows` consecutive rows that start at a multiple of `rows` always lie in one sequence, so that
+  // row_part(first + r) = row_part(first) + r * dim.
+  __device__ __forceinline__ bool rows_share_sequence(int rows) const { return !PAD && seq % rows == 0; }
+  // The same split for the transposed V of the column pass: V^T[b, head, i, s] = vt_col_part(n) + vt_row_part(m),
+  // m the first of eight consecutive rows; whether the eight are one 16-byte store is vt_rows_contiguous(m, limit).
+  __device__ __forceinline__ T* vt_col_part(uint32_t n) const {
+    const uint32_t rem = n - 2 * hidden;
+    return v + (int64_t)rem * v_pitch;  // (head * dim + i) * v_pitch
+  }
+  __device__ __forceinline__ int64_t vt_row_part(int m) const {
+    const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;
+    const uint32_t b = div_seq.div(prow);
+    return (int64_t)b * hidden * v_pitch + (prow - b * seq);
+  }
   __device__ __forceinline__ float finish(float x) const { return x; }
   __device__ __forceinline__ T* dest8(int m, int n) const {  // head_dim % 8 == 0: the eight columns stay in one head
     const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;

@@ -120,8 +120,8 @@ __device__ __forceinline__ S acc_read(S v) {
 // with a wait for ALL outstanding vector memory operations, i.e. also for the global stores of the previous row
 // block, one HBM round trip per block.  The strip is disjoint from the DMA stages, and LDS operations of one
 // wavefront complete in order, so the reads that follow need no more than their usual counter wait.
-__device__ __forceinline__ void strip_write(uint32_t lds_addr, const Chunk& x) {
-  asm volatile("ds_write_b128 %0, %1" : : "v"(lds_addr), "v"(__builtin_bit_cast(Quad, x)) : "memory");
+__device__ __forceinline__ void strip_write(uint32_t lds_addr, Quad x) {
+  asm volatile("ds_write_b128 %0, %1" : : "v"(lds_addr), "v"(x) : "memory");
 }
 
 // Bias of eight consecutive columns, kept in storage precision (16 bytes for 2-byte types) until it is added.
@@ -286,13 +286,13 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   // the output matrix of a linear epilogue: rows at and past M lie outside the resource and their stores are dropped
   const uint32_t ldc_bytes = (uint32_t)LinearDest<Epi>::ldc(epi) * (uint32_t)sizeof(T);
   const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(LinearDest<Epi>::base(epi), 0, (int)min((int64_t)g.m * ldc_bytes, (int64_t)0x7fffffff), 0x00020000);
-  auto store_c = [&](const Chunk& x, uint32_t voff, uint32_t soff) __attribute__((always_inline)) {
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(Quad, x), rsrc_c, (int)voff, (int)soff, 0);
+  auto store_c = [&](Quad x, uint32_t voff, uint32_t soff) __attribute__((always_inline)) {
+    __builtin_amdgcn_raw_buffer_store_b128(x, rsrc_c, (int)voff, (int)soff, 0);
   };
 #else
   auto dma_issue_one = [&](int) {};
   const uint32_t ldc_bytes = 0;
-  auto store_c = [&](const Chunk&, uint32_t, uint32_t) {};
+  auto store_c = [&](Quad, uint32_t, uint32_t) {};
 #endif
   auto dma_issue = [&](auto lo_tag, auto hi_tag) __attribute__((always_inline)) {
     constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
@@ -453,11 +453,22 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
 #pragma unroll
         for (int v = 0; v < NV; ++v) bv[v].widen(bf[v]);
       }
-      const bool whole_width = n0 + BN <= n_lim;  // uniform
-      Chunk landed[PASSES];
+      const bool whole_width = n0 + BN <= n_lim, whole_rows = m0 + BM <= m_lim;  // uniform
+      // epilogues that scatter (the QKV split): the column part of a lane's destinations, once per tile
+      T* col_ptr[PASSES];
+      bool block_in_one_sequence = false;  // uniform: the MF rows of a row block share their batch index
+      if constexpr (!LinearDest<Epi>::value) {
+        block_in_one_sequence = epi.rows_share_sequence(MF);
+#pragma unroll
+        for (int pass = 0; pass < PASSES; ++pass) {
+          col_ptr[pass] = epi.col_part((uint32_t)min(n0 + wn0 + st_col[pass], n_lim - 8));
+          if (block_in_one_sequence) col_ptr[pass] += st_row[pass] * epi.dim;  // the lane's share of the row part
+        }
+      }
+      Quad landed[PASSES];  // first-class vectors: arrays of a struct type may end up in scratch memory
 #pragma unroll
       for (int i = 0; i <= RB; ++i) {
-        Chunk packed[NV];
+        Quad packed[NV];
         if (i < RB) {
 #pragma unroll
           for (int v = 0; v < NV; ++v) {
@@ -477,7 +488,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
             T rounded[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) rounded[e] = from_float<T>(epi.finish(out[e]));
-            packed[v] = pack_chunk(rounded);
+            packed[v] = __builtin_bit_cast(Quad, pack_chunk(rounded));
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -490,10 +501,12 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
               if (whole_width || n0 + wn0 + st_col[pass] < n_lim)
                 store_c(landed[pass], (uint32_t)st_row[pass] * ldc_bytes + (uint32_t)st_col[pass] * (uint32_t)sizeof(T), soff);
           } else {
+            const int64_t block_part = epi.row_part(min(row0, m_lim - 1));  // uniform
 #pragma unroll
             for (int pass = 0; pass < PASSES; ++pass) {
-              const int m = row0 + st_row[pass], ncol = n0 + wn0 + st_col[pass];
-              if (m < m_lim && ncol < n_lim) *reinterpret_cast<Chunk*>(epi.dest8(m, ncol)) = landed[pass];
+              const int m = row0 + st_row[pass];
+              if ((whole_rows || m < m_lim) && (whole_width || n0 + wn0 + st_col[pass] < n_lim))
+                *reinterpret_cast<Quad*>(col_ptr[pass] + (block_in_one_sequence ? block_part : epi.row_part(m))) = landed[pass];
             }
           }
         }
@@ -503,57 +516,87 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
 #pragma unroll
           for (int v = 0; v < NV; ++v) strip_write(strip_lds + (uint32_t)wr_off[v], packed[v]);
 #pragma unroll
-          for (int pass = 0; pass < PASSES; ++pass) landed[pass] = *reinterpret_cast<const Chunk*>(strip + rd_off[pass]);
+          for (int pass = 0; pass < PASSES; ++pass) landed[pass] = *reinterpret_cast<const Quad*>(strip + rd_off[pass]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      W4_STAMP(3)
     } else {
       if constexpr (HasColumnPass<Epi>::value) {
         for (int kt = 0; kt < ksteps; kt += 2) {
           k_step(std::integral_constant<int, 0>{}, std::false_type{});
           k_step(std::integral_constant<int, 1>{}, std::false_type{});
         }
-        // a lane owns column lrow of every block and, after the pair swap, eight consecutive rows of it
+        W4_STAMP(2)
+        // A lane owns column lrow of every block and, after the pair swap, eight consecutive rows of it: one 16-byte
+        // piece of a V^T row.  Stored as they lie, the 64 lanes of an instruction would touch 64 different rows of
+        // V^T.  So the pieces of 32 columns x 64 rows go through the wavefront's strip ([column][64 rows], column
+        // pitch 144 bytes: the 16 lanes the LDS serves together land in 16 different 16-byte slots) and come back with
+        // eight adjacent lanes holding the 128 contiguous bytes of one column.  As in the row path, the arithmetic
+        // of unit u runs while the strip reads of unit u-1 are in flight.
+        constexpr int VT_PITCH = 144, UNITS = CB * 2, VP = 4;  // unit = (block column j, half of the 128 rows)
+        static_assert(32 * VT_PITCH <= MF * PITCH, "the transposed unit fits the strip");
         float bj[CB];
         load_bias_columns_stride<CB, MF>(epi, n0 + wn0 + lrow, n_lim, bj);
+        const int rd_col = lane >> 3, rd_chunk = lane & 7;  // pass p returns rows 8*rd_chunk.. of column 8*p + rd_col
+        const bool rows_whole = m0 + BM <= m_lim && epi.seq % 8 == 0;  // uniform: every group of eight is one store
+        T* const vt_base = epi.vt_col_part((uint32_t)min(n0 + wn0 + rd_col, n_lim - 1));
+        Quad vt_landed[VP];
 #pragma unroll
-        for (int j = 0; j < CB; ++j) {
-          const int ncol = n0 + wn0 + j * MF + lrow;
-          if constexpr (MF == 32) {
+        for (int u = 0; u <= UNITS; ++u) {
+          Quad piece[4];
+          if (u < UNITS) {
+            const int j = u / 2, hf = u % 2;
 #pragma unroll
-            for (int i = 0; i < RB; ++i)
-#pragma unroll
-              for (int gp = 0; gp < 2; ++gp) {
-                float out[8];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                  float a = acc[i][j][8 * gp + e], b = acc[i][j][8 * gp + 4 + e];
-                  pair_swap<32>(a, b);
-                  out[e] = a + bj[j];
-                  out[4 + e] = b + bj[j];
-                }
-                const int m = m0 + wm0 + i * 32 + 16 * gp + 8 * lgrp;
-                if (m < m_lim && ncol < n_lim) epi.store_col8(m, m_lim, ncol, out);
-              }
-          } else {
-#pragma unroll
-            for (int i = 0; i < RB; i += 2) {
+            for (int q = 0; q < 4; ++q) {
+              const int i = 2 * hf + q / 2, gp = q % 2;
               float out[8];
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
-                float a = acc[i][j][e], b = acc[i + 1][j][e];
-                pair_swap<16>(a, b);
+                float a = acc_read(acc[i][j][8 * gp + e]), b = acc_read(acc[i][j][8 * gp + 4 + e]);
+                pair_swap<32>(a, b);
                 out[e] = a + bj[j];
                 out[4 + e] = b + bj[j];
               }
-              const int m = m0 + wm0 + (i + (lgrp & 1)) * 16 + 8 * (lgrp >> 1);
-              if (m < m_lim && ncol < n_lim) epi.store_col8(m, m_lim, ncol, out);
+              T rounded[8];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) rounded[e] = from_float<T>(out[e]);
+              piece[q] = __builtin_bit_cast(Quad, pack_chunk(rounded));
             }
           }
+          __builtin_amdgcn_sched_barrier(0);
+          if (u > 0) {
+            const int j = (u - 1) / 2, hf = (u - 1) % 2;
+            const int m = m0 + wm0 + hf * 64 + rd_chunk * 8;
+            const int64_t row_off = epi.vt_row_part(min(m, m_lim - 1));
+#pragma unroll
+            for (int p = 0; p < VP; ++p) {
+              const int ncol = n0 + wn0 + j * MF + p * 8 + rd_col;
+              T* dst = vt_base + (int64_t)(j * MF + p * 8) * epi.v_pitch + row_off;
+              if (rows_whole) {
+                if (ncol < n_lim) *reinterpret_cast<Quad*>(dst) = vt_landed[p];
+              } else if (m < m_lim && ncol < n_lim) {
+                const Vec<T, 8> x = __builtin_bit_cast(Vec<T, 8>, vt_landed[p]);
+                float out[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) out[e] = to_float(x.v[e]);
+                epi.store_col8(m, m_lim, ncol, out);
+              }
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (u < UNITS) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              strip_write(strip_lds + (uint32_t)(lrow * VT_PITCH + ((q / 2) * 4 + (q % 2) * 2 + lgrp) * 16), piece[q]);
+#pragma unroll
+            for (int p = 0; p < VP; ++p)
+              vt_landed[p] = *reinterpret_cast<const Quad*>(strip + (p * 8 + rd_col) * VT_PITCH + rd_chunk * 16);
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
+    W4_STAMP(3)
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // surplus DMA loads have landed before the LDS is given back
 }
@@ -623,6 +666,17 @@ struct LargeTileKernel<T, EpiBias<T, ACT, HAS_ACT, false>, typename std::enable_
       if (force == nullptr || force[0] != '1') return false;
     }
     return w4_output_fits<T>(g, epi.ldc) && w4_wanted<T>(g, epi, batch, aligned);
+  }
+  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
+};
+// Bias + head split of a dense (not packed) batch.  With V kept transposed the tiles of the V third run unswapped, so
+// that third has to start on a tile boundary.
+template <typename T>
+struct LargeTileKernel<T, EpiQkvSplit<T, false>, typename std::enable_if<sizeof(T) == 2>::type> {
+  using Epi = EpiQkvSplit<T, false>;
+  static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
+    if (epi.v_pitch > 0 && (2 * epi.hidden) % 192 != 0) return false;
+    return w4_wanted<T>(g, epi, batch, aligned);
   }
   static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
 };

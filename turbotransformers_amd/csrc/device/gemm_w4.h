@@ -67,15 +67,21 @@ struct MmaBlock<int8_t, 32> {
 template <>
 struct MmaBlock<f16, 16> {
   using Acc = floatx4;
+  // Written as an instruction with the accumulator pinned to the AGPR half ("+a"): through the builtin the compiler
+  // keeps part of the 192 accumulator registers of the 16-wide blocks in ordinary registers and moves them back and
+  // forth around every matrix instruction (two copies per MFMA in the K loop).
   static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
-    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(__builtin_bit_cast(halfx8, a)), "v"(__builtin_bit_cast(halfx8, b)));
   }
 };
 template <>
 struct MmaBlock<bf16, 16> {
   using Acc = floatx4;
+  // Written as an instruction with the accumulator pinned to the AGPR half ("+a"): through the builtin the compiler
+  // keeps part of the 192 accumulator registers of the 16-wide blocks in ordinary registers and moves them back and
+  // forth around every matrix instruction (two copies per MFMA in the K loop).
   static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
-    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(__builtin_bit_cast(bf16x8, a)), "v"(__builtin_bit_cast(bf16x8, b)));
   }
 };
 template <>
@@ -159,6 +165,10 @@ struct BiasVec {
 };
 
 constexpr int kW4Threads = 256;
+// Block size of the matrix instruction the launchers use: 16 (v_mfma_f32_16x16x32) moves a quarter of the accumulator
+// bits per FLOP of the 32x32x16 form, and on a chip that runs its matrix loops at the power limit that is clock rate:
+// the same K loop runs 5-10 % faster with it.
+constexpr int kW4Block = 16;
 
 // Epilogues whose output is one row-major matrix: base address and leading dimension, so that the kernel can
 // store through a buffer resource (32-bit offsets, rows past M dropped by the hardware's range check).
@@ -194,14 +204,14 @@ __device__ unsigned long long w4_trace[4][16][8][2];
 template <int BN, int MF>
 constexpr int w4_strip_pitch() { return BN == 256 ? 256 : BN + 16; }  // bytes per staged row (BN/2 columns of 2 bytes)
 template <int BN, int MF>
-constexpr int w4_lds_bytes() { return 2 * (256 + BN) * kRowBytes + 4 * MF * w4_strip_pitch<BN, MF>(); }
+constexpr int w4_lds_bytes() { return 2 * (256 + BN) * kRowBytes + 4 * 32 * w4_strip_pitch<BN, MF>(); }
 
 // What the kernel needs from an epilogue besides bias_ptr(): finish(x) applied to acc + bias in fp32, and
 // dest8(m, n), the address of the 16 bytes that hold columns n..n+7 of output row m.
 template <typename T, int BN, int MF, typename Epi>
 __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, const Epi epi) {
   static_assert(sizeof(T) == 2, "16-bit operands");
-  static_assert(MF == 32, "the epilogue pairs lanes l and l + 32");
+  static_assert(MF == 32 || MF == 16, "block sizes of the matrix instructions");
   constexpr int BM = 256;
   constexpr int BK = kRowBytes / sizeof(T);
   constexpr int RB = 128 / MF, CB = BN / 2 / MF;   // blocks per wavefront: rows, columns
@@ -383,7 +393,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   dma_issue(std::integral_constant<int, 0>{}, std::integral_constant<int, D3>{});
   read_frags(0, 0, fa[0], fb[0]);
 
-  char* strip = smem + 2 * STAGE + wave * (MF * PITCH);
+  char* strip = smem + 2 * STAGE + wave * (32 * PITCH);
   const uint32_t strip_lds = (uint32_t)reinterpret_cast<uintptr_t>(strip);  // low half of a generic LDS address = LDS offset
   int tile = first;
   for (int t = 0; t < my_tiles; ++t, tile += stride) {
@@ -405,11 +415,19 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     using BiasT = typename std::remove_cv<typename std::remove_pointer<decltype(bias)>::type>::type;
     const int m_lim = g.m, n_lim = g.n;
     // bias of this lane's column groups, requested now so that it has landed when the epilogue wants it
-    constexpr int NV = CB * 2;
-    BiasVec<BiasT> bv[NV];
+    // The epilogue works on groups of 32 rows; a lane contributes NV units of eight consecutive columns to each.
+    // MF = 32: unit v = (block column v/2, half v%2 of its 32 columns), the lane's row is lrow.  MF = 16: unit v =
+    // (16-row block v / (CB/2) of the pair, pair of block columns v % (CB/2)), the lane's row is 16*(v / (CB/2)) + lrow.
+    constexpr int NV = MF == 32 ? CB * 2 : CB;
+    constexpr int NBV = MF == 32 ? NV : CB / 2;  // distinct column groups among the units (= bias vectors to hold)
+    auto unit_chunk = [&](int v) __attribute__((always_inline)) {  // which group of eight columns of the wavefront's BN/2
+      if constexpr (MF == 32) return (v / 2) * 4 + (v % 2) * 2 + lgrp;
+      else return 2 * (2 * (v % (CB / 2)) + (lgrp & 1)) + (lgrp >> 1);
+    };
+    BiasVec<BiasT> bv[NBV];
     if (swap) {
 #pragma unroll
-      for (int v = 0; v < NV; ++v) bv[v].load(bias, min(n0 + wn0 + ((v / 2) * 4 + (v % 2) * 2 + lgrp) * 8, n_lim - 8), g.b);  // N % 8 == 0
+      for (int v = 0; v < NBV; ++v) bv[v].load(bias, min(n0 + wn0 + unit_chunk(v) * 8, n_lim - 8), g.b);  // N % 8 == 0
     }
     W4_STAMP(1)
     if (swap) {
@@ -431,8 +449,9 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       // bytes per lane.  A lone wavefront on a SIMD hides no latency by itself, so the order is written out: the
       // arithmetic of row block i runs while the strip reads of block i-1 are in flight, then the stores of block
       // i-1 go out back to back, then block i is written to the strip and its reads are issued.
-      constexpr int PASSES = MF * CPR / kWave;
-      static_assert(MF * CPR % kWave == 0, "whole passes over a strip");
+      constexpr int GROUP = 32, GROUPS = 128 / GROUP;  // rows staged at a time
+      constexpr int PASSES = GROUP * CPR / kWave;
+      static_assert(GROUP * CPR % kWave == 0, "whole passes over a strip");
       int rd_off[PASSES], st_row[PASSES], st_col[PASSES], wr_off[NV];
 #pragma unroll
       for (int pass = 0; pass < PASSES; ++pass) {
@@ -444,21 +463,21 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       }
 #pragma unroll
       for (int v = 0; v < NV; ++v) {
-        const int c = (v / 2) * 4 + (v % 2) * 2 + lgrp;
-        wr_off[v] = lrow * PITCH + ((XOR_STRIP ? (c ^ (lrow & (CPR - 1))) : c) << 4);
+        const int c = unit_chunk(v), row = MF == 32 ? lrow : 16 * (v / (CB / 2)) + lrow;
+        wr_off[v] = row * PITCH + ((XOR_STRIP ? (c ^ (row & (CPR - 1))) : c) << 4);
       }
-      float bf[NV][8];
+      float bf[NBV][8];
       const bool has_bias = bias != nullptr;  // uniform
       if (has_bias) {
 #pragma unroll
-        for (int v = 0; v < NV; ++v) bv[v].widen(bf[v]);
+        for (int v = 0; v < NBV; ++v) bv[v].widen(bf[v]);
       }
       const bool whole_width = n0 + BN <= n_lim, whole_rows = m0 + BM <= m_lim;  // uniform
       // epilogues that scatter (the QKV split): the column part of a lane's destinations, once per tile
       T* col_ptr[PASSES];
-      bool block_in_one_sequence = false;  // uniform: the MF rows of a row block share their batch index
+      bool block_in_one_sequence = false;  // uniform: the rows of a group share their batch index
       if constexpr (!LinearDest<Epi>::value) {
-        block_in_one_sequence = epi.rows_share_sequence(MF);
+        block_in_one_sequence = epi.rows_share_sequence(GROUP);
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
           col_ptr[pass] = epi.col_part((uint32_t)min(n0 + wn0 + st_col[pass], n_lim - 8));
@@ -467,23 +486,29 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       }
       Quad landed[PASSES];  // first-class vectors: arrays of a struct type may end up in scratch memory
 #pragma unroll
-      for (int i = 0; i <= RB; ++i) {
+      for (int i = 0; i <= GROUPS; ++i) {
         Quad packed[NV];
-        if (i < RB) {
+        if (i < GROUPS) {
 #pragma unroll
           for (int v = 0; v < NV; ++v) {
-            const int j = v / 2, gp = v % 2;
             float out[8];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              float a = acc_read(acc[i][j][8 * gp + e]), b = acc_read(acc[i][j][8 * gp + 4 + e]);
-              pair_swap<32>(a, b);
+              float a, b;
+              if constexpr (MF == 32) {
+                a = acc_read(acc[i][v / 2][8 * (v % 2) + e]);
+                b = acc_read(acc[i][v / 2][8 * (v % 2) + 4 + e]);
+              } else {
+                a = acc_read(acc[2 * i + v / (CB / 2)][2 * (v % (CB / 2))][e]);
+                b = acc_read(acc[2 * i + v / (CB / 2)][2 * (v % (CB / 2)) + 1][e]);
+              }
+              pair_swap<MF>(a, b);
               out[e] = a;
               out[4 + e] = b;
             }
             if (has_bias) {
 #pragma unroll
-              for (int e = 0; e < 8; ++e) out[e] += bf[v][e];
+              for (int e = 0; e < 8; ++e) out[e] += bf[v % NBV][e];
             }
             T rounded[8];
 #pragma unroll
@@ -493,7 +518,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
         }
         __builtin_amdgcn_sched_barrier(0);
         if (i > 0) {
-          const int row0 = m0 + wm0 + (i - 1) * MF;
+          const int row0 = m0 + wm0 + (i - 1) * GROUP;
           if constexpr (LinearDest<Epi>::value) {
             const uint32_t soff = (uint32_t)row0 * ldc_bytes + (uint32_t)(n0 + wn0) * (uint32_t)sizeof(T);
 #pragma unroll
@@ -511,7 +536,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
           }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (i < RB) {
+        if (i < GROUPS) {
           // same wavefront, LDS operations complete in order: no barrier between the writes and the reads
 #pragma unroll
           for (int v = 0; v < NV; ++v) strip_write(strip_lds + (uint32_t)wr_off[v], packed[v]);
@@ -533,8 +558,8 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
         // pitch 144 bytes: the 16 lanes the LDS serves together land in 16 different 16-byte slots) and come back with
         // eight adjacent lanes holding the 128 contiguous bytes of one column.  As in the row path, the arithmetic
         // of unit u runs while the strip reads of unit u-1 are in flight.
-        constexpr int VT_PITCH = 144, UNITS = CB * 2, VP = 4;  // unit = (block column j, half of the 128 rows)
-        static_assert(32 * VT_PITCH <= MF * PITCH, "the transposed unit fits the strip");
+        constexpr int VT_PITCH = 144, UNITS = (BN / 2 / 32) * 2, VP = 4;  // unit = (32 columns, half of the 128 rows)
+        static_assert(32 * VT_PITCH <= 32 * PITCH, "the transposed unit fits the strip");
         float bj[CB];
         load_bias_columns_stride<CB, MF>(epi, n0 + wn0 + lrow, n_lim, bj);
         const int rd_col = lane >> 3, rd_chunk = lane & 7;  // pass p returns rows 8*rd_chunk.. of column 8*p + rd_col
@@ -545,17 +570,25 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
         for (int u = 0; u <= UNITS; ++u) {
           Quad piece[4];
           if (u < UNITS) {
-            const int j = u / 2, hf = u % 2;
+            const int j = u / 2, hf = u % 2;  // columns 32j.., rows 64hf..
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              const int i = 2 * hf + q / 2, gp = q % 2;
               float out[8];
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
-                float a = acc_read(acc[i][j][8 * gp + e]), b = acc_read(acc[i][j][8 * gp + 4 + e]);
-                pair_swap<32>(a, b);
-                out[e] = a + bj[j];
-                out[4 + e] = b + bj[j];
+                float a, b, bias_q;
+                if constexpr (MF == 32) {  // piece q: rows 32*(q/2) + 16*(q%2) + 8*lgrp.. of column lrow
+                  a = acc_read(acc[2 * hf + q / 2][j][8 * (q % 2) + e]);
+                  b = acc_read(acc[2 * hf + q / 2][j][8 * (q % 2) + 4 + e]);
+                  bias_q = bj[j];
+                } else {  // piece q: column 16*(q/2) + lrow, rows 32*(q%2) + 16*(lgrp&1) + 8*(lgrp>>1)..
+                  a = acc_read(acc[4 * hf + 2 * (q % 2)][2 * j + q / 2][e]);
+                  b = acc_read(acc[4 * hf + 2 * (q % 2) + 1][2 * j + q / 2][e]);
+                  bias_q = bj[2 * j + q / 2];
+                }
+                pair_swap<MF>(a, b);
+                out[e] = a + bias_q;
+                out[4 + e] = b + bias_q;
               }
               T rounded[8];
 #pragma unroll
@@ -570,8 +603,8 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
             const int64_t row_off = epi.vt_row_part(min(m, m_lim - 1));
 #pragma unroll
             for (int p = 0; p < VP; ++p) {
-              const int ncol = n0 + wn0 + j * MF + p * 8 + rd_col;
-              T* dst = vt_base + (int64_t)(j * MF + p * 8) * epi.v_pitch + row_off;
+              const int ncol = n0 + wn0 + j * 32 + p * 8 + rd_col;
+              T* dst = vt_base + (int64_t)(j * 32 + p * 8) * epi.v_pitch + row_off;
               if (rows_whole) {
                 if (ncol < n_lim) *reinterpret_cast<Quad*>(dst) = vt_landed[p];
               } else if (m < m_lim && ncol < n_lim) {
@@ -586,8 +619,12 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
           __builtin_amdgcn_sched_barrier(0);
           if (u < UNITS) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-              strip_write(strip_lds + (uint32_t)(lrow * VT_PITCH + ((q / 2) * 4 + (q % 2) * 2 + lgrp) * 16), piece[q]);
+            for (int q = 0; q < 4; ++q) {
+              // [column of the unit][group of eight rows of the half]
+              const int col = MF == 32 ? lrow : 16 * (q / 2) + lrow;
+              const int rows8 = MF == 32 ? (q / 2) * 4 + (q % 2) * 2 + lgrp : (q % 2) * 4 + (lgrp & 1) * 2 + (lgrp >> 1);
+              strip_write(strip_lds + (uint32_t)(col * VT_PITCH + rows8 * 16), piece[q]);
+            }
 #pragma unroll
             for (int p = 0; p < VP; ++p)
               vt_landed[p] = *reinterpret_cast<const Quad*>(strip + (p * 8 + rd_col) * VT_PITCH + rd_chunk * 16);
@@ -619,7 +656,7 @@ static bool w4_output_fits(const GemmArgs& g, int64_t ldc) {
 
 template <typename T, int BN, typename Epi>
 static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s) {
-  constexpr int LDS = w4_lds_bytes<BN, 32>();
+  constexpr int LDS = w4_lds_bytes<BN, kW4Block>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
   if (describe_only("dma_agpr", 4, 256, BN)) return 0;
   g.tiles_m = (g.m + 255) / 256;
@@ -628,7 +665,7 @@ static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s) {
   TTMI_REQUIRE(tiles < (1ll << 30), "GEMM grid too large");
   // one persistent workgroup per CU (the LDS allows no second one), a multiple of the XCD count
   const unsigned grid = (unsigned)(std::min<int64_t>(ceil_div(tiles, kNumXcd), std::max(1, compute_units() / kNumXcd)) * kNumXcd);
-  auto kern = gemm_w4_kernel<T, BN, 32, Epi>;
+  auto kern = gemm_w4_kernel<T, BN, kW4Block, Epi>;
   const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
   if (rc != 0) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kW4Threads), LDS, s, g, epi);
@@ -654,17 +691,12 @@ static bool w4_wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned
 }
 
 // Bias, and bias + activation.  With an activation the epilogue is a long stretch of VALU work (two transcendentals
-// per element) that nothing overlaps when a SIMD holds a single wavefront: inside the encoder the FFN1 product
-// (N = 3072, K = 768: twelve K steps per tile) ran 2.6 % slower here than on the 8-wavefront kernel, so those
-// problems come here only when forced.
+// per element: about a third of the FFN1 product's time) that nothing overlaps when a SIMD holds a single wavefront;
+// the 8-wavefront kernel pays the same arithmetic, so the faster K loop still decides.
 template <typename T, int ACT, bool HAS_ACT>
 struct LargeTileKernel<T, EpiBias<T, ACT, HAS_ACT, false>, typename std::enable_if<sizeof(T) == 2>::type> {
   using Epi = EpiBias<T, ACT, HAS_ACT, false>;
   static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
-    if (HAS_ACT) {
-      const char* force = std::getenv("TTMI_LARGE_TILE");
-      if (force == nullptr || force[0] != '1') return false;
-    }
     return w4_output_fits<T>(g, epi.ldc) && w4_wanted<T>(g, epi, batch, aligned);
   }
   static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }

@@ -267,6 +267,37 @@ PYBIND11_MODULE(turbo_transformers_cxx, m) {
            "input_ids int64 [B,S] on the GPU -> last hidden state [B,S,H]; the whole forward in C++");
 
   // ---- additions of this build --------------------------------------------------------------
+  // The layer loop of an encoder in one call: hidden -> [attention -> intermediate -> output] x layers -> out.  What the
+  // Python BertEncoder does layer by layer, without a round trip through the interpreter per sub-layer (three calls,
+  // three temporaries and a stream query each: at batch 1 x seq 128 the interpreter, not the GPU, set the pace).
+  // `layer_list` is a sequence of (BertAttention, BertIntermediate, BertOutput).  No counterpart in the reference.
+  m.def("run_bert_layers", [](const py::sequence& layer_list, const Tensor& hidden, const Tensor& mask, Tensor* out) {
+    struct Sub {
+      const layers::BertAttention* attention;
+      const layers::BertIntermediate* intermediate;
+      const layers::BertOutput* output;
+    };
+    std::vector<Sub> subs;
+    subs.reserve(py::len(layer_list));
+    for (const py::handle& item : layer_list) {
+      const py::tuple t = py::cast<py::tuple>(item);
+      TT_ENFORCE_EQ(py::len(t), (size_t)3, "each layer is (attention, intermediate, output)");
+      subs.push_back(Sub{&py::cast<const layers::BertAttention&>(t[0]), &py::cast<const layers::BertIntermediate&>(t[1]),
+                         &py::cast<const layers::BertOutput&>(t[2])});
+    }
+    TT_ENFORCE(!subs.empty() && out != nullptr, "run_bert_layers needs layers and an output tensor");
+    Tensor attention_out(nullptr), intermediate_out(nullptr), even(nullptr), odd(nullptr);
+    const Tensor* current = &hidden;
+    for (size_t i = 0; i < subs.size(); ++i) {
+      // the last layer writes the caller's tensor; before it two buffers alternate (a layer never writes what it reads)
+      Tensor* target = (i + 1 == subs.size()) ? out : (i % 2 == 0 ? &even : &odd);
+      (*subs[i].attention)(*current, mask, &attention_out, nullptr, false);
+      (*subs[i].intermediate)(attention_out, &intermediate_out);
+      (*subs[i].output)(intermediate_out, attention_out, target);
+      current = target;
+    }
+  });
+
   m.def("set_stream", [](uintptr_t s) { core::DeviceContext::GetInstance().set_stream(reinterpret_cast<void*>(s)); },
         "Enqueue all following kernels on this hipStream_t (pass torch.cuda.current_stream().cuda_stream).");
   m.def("synchronize", [] { core::DeviceContext::GetInstance().Wait(); },

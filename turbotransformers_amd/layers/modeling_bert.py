@@ -170,6 +170,13 @@ class BertEncoder:
         all_hidden_states, all_attentions = (), ()
         hidden_states = try_convert(hidden_states)
         attention_mask = try_convert(attention_mask)
+        if not output_attentions and not output_hidden_states and self._plain_layers():
+            # nothing but the last hidden state is asked for: the layer loop runs inside the extension
+            use_current_stream()
+            last = cxx.Tensor.create_empty()
+            cxx.run_bert_layers([(l.attention, l.intermediate, l.output) for l in self.layer], hidden_states,
+                                create_empty_if_none(attention_mask), last)
+            return (convert_returns_as_type(last, return_type), )
         for layer in self.layer:
             layer_outputs = layer(hidden_states=hidden_states, attention_mask=attention_mask,
                                   output_attentions=output_attentions, return_type=ReturnType.turbo_transformers)
@@ -185,6 +192,12 @@ class BertEncoder:
         if output_attentions:
             outputs = outputs + (all_attentions, )
         return outputs
+
+    def _plain_layers(self):
+        """Whether every layer is a BertLayer built from the three stock sub-layers (then the C++ loop may run them)."""
+        return len(self.layer) > 0 and all(
+            type(l) is BertLayer and type(l.attention) is BertAttention and type(l.intermediate) is BertIntermediate
+            and type(l.output) is BertOutput for l in self.layer)
 
     @staticmethod
     def from_torch(encoder):

@@ -136,6 +136,9 @@ struct GemmArgs {
   int64_t a_outer, a_inner, b_outer, b_inner;
   int tiles_m, tiles_n;
   int k_chunk;  // split-K: blockIdx.y owns K range [y*k_chunk, (y+1)*k_chunk) and z passed to the epilogue is y; 0 = whole K
+  // One-wavefront-per-SIMD kernel only: a column at which a new run of tiles starts (0 = none).  Tile columns
+  // [0, split_tiles) cover [0, split_col), the last of them ragged; the tiles after them start at split_col again.
+  int split_col, split_tiles;
 };
 
 // ------------------------------------------------------------------------ epilogues -----

@@ -257,13 +257,17 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   //      chunk l%8 of row l/8 and therefore fetches logical chunk (l%8) ^ ((row>>1)&7).  The LOADS loads of one K
   //      step are not issued as a burst: the memory pipeline takes about 20 cycles per load and serves the four
   //      wavefronts in turn, and a wavefront that finds its queue full stops issuing MFMAs.
+  // first column of tile column tile_n: a second run of tiles may start at g.split_col (see GemmArgs)
+  auto first_column = [&](int tile_n) __attribute__((always_inline)) {
+    return tile_n < g.split_tiles ? tile_n * BN : g.split_col + (tile_n - g.split_tiles) * BN;
+  };
   int dma_step = 0, dma_k = 0, dma_tile = first;
   uint32_t voa[A_LOADS], vob[B_LOADS];  // per-lane byte offsets from the tile's first row (row clamp and swizzle inside)
   uint32_t a_soff = 0, b_soff = 0;  // byte offset of the cursor's tile in A and in B (matrices below 2 GiB, checked by the launcher)
   auto dma_point = [&](int tile) __attribute__((always_inline)) {
     int tile_m, tile_n;
     tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = tile_m * BM, n0 = first_column(tile_n);
     const int sub = lane >> 3, p = lane & 7;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
@@ -399,7 +403,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   for (int t = 0; t < my_tiles; ++t, tile += stride) {
     int tile_m, tile_n;
     tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = tile_m * BM, n0 = first_column(tile_n);
     bool swap = true;
     if constexpr (HasColumnPass<Epi>::value) swap = !(epi.column_pass() && n0 >= epi.first_column_of_pass());
     W4_STAMP(0)
@@ -413,7 +417,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
 
     const auto* bias = epi.bias_ptr();
     using BiasT = typename std::remove_cv<typename std::remove_pointer<decltype(bias)>::type>::type;
-    const int m_lim = g.m, n_lim = g.n;
+    const int m_lim = g.m, n_lim = tile_n < g.split_tiles ? g.split_col : g.n;  // a tile in front of the split ends there
     // bias of this lane's column groups, requested now so that it has landed when the epilogue wants it
     // The epilogue works on groups of 32 rows; a lane contributes NV units of eight consecutive columns to each.
     // MF = 32: unit v = (block column v/2, half v%2 of its 32 columns), the lane's row is lrow.  MF = 16: unit v =
@@ -466,9 +470,12 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
         const int c = unit_chunk(v), row = MF == 32 ? lrow : 16 * (v / (CB / 2)) + lrow;
         wr_off[v] = row * PITCH + ((XOR_STRIP ? (c ^ (row & (CPR - 1))) : c) << 4);
       }
-      float bf[NBV][8];
+      // The bias is widened to fp32 once per tile when that costs at most 24 registers; the widest tile keeps it in
+      // storage precision and widens eight values at each use instead (its epilogue has no registers to spare).
+      constexpr bool WIDE_BIAS = NBV * 8 <= 24;
+      float bf[WIDE_BIAS ? NBV : 1][8];
       const bool has_bias = bias != nullptr;  // uniform
-      if (has_bias) {
+      if (WIDE_BIAS && has_bias) {
 #pragma unroll
         for (int v = 0; v < NBV; ++v) bv[v].widen(bf[v]);
       }
@@ -507,8 +514,12 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
               out[4 + e] = b;
             }
             if (has_bias) {
+              if constexpr (WIDE_BIAS) {
 #pragma unroll
-              for (int e = 0; e < 8; ++e) out[e] += bf[v % NBV][e];
+                for (int e = 0; e < 8; ++e) out[e] += bf[v % NBV][e];
+              } else {
+                bv[v % NBV].add_to(out);
+              }
             }
             T rounded[8];
 #pragma unroll
@@ -634,6 +645,11 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       }
     }
     W4_STAMP(3)
+    // The last substep of the K loop has already fetched the first fragments of the next tile.  Fetching them again
+    // here (K step 0 of the next tile sits untouched in stage 0 until that tile's own loads overwrite it) ends the
+    // life of those registers at the end of the K loop, so the epilogue has them: up to 64 with 16-wide blocks.
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(0, 0, fa[0], fb[0]);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // surplus DMA loads have landed before the LDS is given back
 }
@@ -654,13 +670,16 @@ static bool w4_output_fits(const GemmArgs& g, int64_t ldc) {
   return (int64_t)g.m * ldc * (int64_t)sizeof(T) < ((int64_t)1 << 31);
 }
 
+// split_col: a column (multiple of 8) at which a fresh tile has to start whatever BN is (0 = none).
 template <typename T, int BN, typename Epi>
-static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s) {
+static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s, int split_col = 0) {
   constexpr int LDS = w4_lds_bytes<BN, kW4Block>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
   if (describe_only("dma_agpr", 4, 256, BN)) return 0;
   g.tiles_m = (g.m + 255) / 256;
-  g.tiles_n = (g.n + BN - 1) / BN;
+  g.split_col = split_col;
+  g.split_tiles = split_col > 0 ? (split_col + BN - 1) / BN : 0;
+  g.tiles_n = g.split_tiles + (g.n - split_col + BN - 1) / BN;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
   TTMI_REQUIRE(tiles < (1ll << 30), "GEMM grid too large");
   // one persistent workgroup per CU (the LDS allows no second one), a multiple of the XCD count
@@ -675,6 +694,10 @@ static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s) {
 // The 256 x 192 tile against the tile configurations of the 8-wavefront kernels: the same cost model, with the
 // efficiency this kernel measured against them on the encoder shapes.
 constexpr TileConfig kW4Tile192{256, 192, 1, 1.06f};
+// The 256 x 256 tile of the same kernel (all 256 AGPRs of a lane are accumulators): a quarter fewer LDS fragment reads
+// and DMA bytes per FLOP, for widths that 192 does not divide well (1024 and 4096 of the BERT-large shapes).  Only the
+// epilogues with one row-major output have it; the head split needs more registers than are left.
+constexpr TileConfig kW4Tile256{256, 256, 1, 1.10f};
 
 // TTMI_LARGE_TILE=0 keeps every problem on the 8-wavefront kernels, =1 sends every eligible problem here whatever
 // the cost model says (for A/B timing and for tests of small and ragged shapes); unset: the cost model decides.
@@ -687,7 +710,15 @@ static bool w4_wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned
   }
   double other = 0;
   (void)pick_tile(g.m, g.n, batch, &other);
-  return tile_cost(kW4Tile192, g.m, g.n, batch) < other;
+  const double mine = LinearDest<Epi>::value ? std::min(tile_cost(kW4Tile192, g.m, g.n, batch), tile_cost(kW4Tile256, g.m, g.n, batch))
+                                             : tile_cost(kW4Tile192, g.m, g.n, batch);
+  return mine < other;
+}
+// Which of the two tile widths a linear epilogue takes.
+template <typename T, typename Epi>
+static int launch_w4_linear(const GemmArgs& g, const Epi& epi, hipStream_t s) {
+  if (tile_cost(kW4Tile256, g.m, g.n, 1) < tile_cost(kW4Tile192, g.m, g.n, 1)) return launch_w4<T, 256>(g, epi, s);
+  return launch_w4<T, 192>(g, epi, s);
 }
 
 // Bias, and bias + activation.  With an activation the epilogue is a long stretch of VALU work (two transcendentals
@@ -699,18 +730,30 @@ struct LargeTileKernel<T, EpiBias<T, ACT, HAS_ACT, false>, typename std::enable_
   static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
     return w4_output_fits<T>(g, epi.ldc) && w4_wanted<T>(g, epi, batch, aligned);
   }
-  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
+  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4_linear<T>(g, epi, s); }
 };
 // Bias + head split of a dense (not packed) batch.  With V kept transposed the tiles of the V third run unswapped, so
-// that third has to start on a tile boundary.
+// that third starts on a tile boundary: where 2 * hidden is no multiple of the tile width, the tile in front of it is
+// cut short and a new run of tiles begins (GemmArgs::split_col).
 template <typename T>
 struct LargeTileKernel<T, EpiQkvSplit<T, false>, typename std::enable_if<sizeof(T) == 2>::type> {
   using Epi = EpiQkvSplit<T, false>;
-  static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
-    if (epi.v_pitch > 0 && (2 * epi.hidden) % 192 != 0) return false;
-    return w4_wanted<T>(g, epi, batch, aligned);
+  // a transposed V third that does not start on a multiple of the tile width starts a run of tiles of its own
+  static bool split_run(const GemmArgs& g, const Epi& epi) {
+    return epi.v_pitch > 0 && g.n == 3 * epi.hidden && (2 * epi.hidden) % 192 != 0;
   }
-  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
+  static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
+    if (!w4_wanted<T>(g, epi, batch, aligned)) return false;
+    if (!split_run(g, epi) || std::getenv("TTMI_LARGE_TILE") != nullptr) return true;
+    // the cost model again, with the tile columns the two runs really have (one or two of them ragged)
+    const int64_t columns = ceil_div(2 * epi.hidden, 192) + ceil_div(epi.hidden, 192);
+    double other = 0;
+    (void)pick_tile(g.m, g.n, batch, &other);
+    return tile_cost(kW4Tile192, g.m, columns * 192, batch) < other;
+  }
+  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) {
+    return launch_w4<T, 192>(g, epi, s, split_run(g, epi) ? 2 * epi.hidden : 0);
+  }
 };
 template <typename T>
 struct LargeTileKernel<T, EpiAlphaBeta<T>, typename std::enable_if<sizeof(T) == 2>::type> {
@@ -718,7 +761,7 @@ struct LargeTileKernel<T, EpiAlphaBeta<T>, typename std::enable_if<sizeof(T) == 
   static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
     return epi.beta == 0.f && w4_output_fits<T>(g, epi.ldc) && w4_wanted<T>(g, epi, batch, aligned);
   }
-  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4<T, 192>(g, epi, s); }
+  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) { return launch_w4_linear<T>(g, epi, s); }
 };
 
 }  // namespace ttmi

@@ -145,7 +145,8 @@ def test_large_tile_kernel_against_oracle_and_small_tiles(ttmi, oracle, large_ti
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
 @pytest.mark.parametrize("v_transposed", [False, True])
-@pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 100, 6, 64), (2, 300, 16, 64), (64, 32, 12, 64)])
+@pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 100, 6, 64), (2, 300, 16, 64), (64, 32, 12, 64),
+                                     (20, 512, 16, 64)])
 def test_large_tile_kernel_qkv_split(ttmi, oracle, large_tile_forced, dt, B, S, h, d, v_transposed):
     """The same kernel behind the QKV projection: bias + head split, V row-major or transposed (those tiles run with
     the matrix operands unswapped and leave through the strip column-wise).  Sequence lengths that are and are not
@@ -166,6 +167,8 @@ def test_large_tile_kernel_qkv_split(ttmi, oracle, large_tile_forced, dt, B, S, 
     name = ctypes.create_string_buffer(64)
     ok(ttmi.ttmi_gemm_describe(B * S, 3 * H, H, capi.EPI_QKV_SPLIT, ctypes.byref(args), TTMI_DTYPES[dt], name, 64))
     assert name.value.decode().startswith("dma_agpr4w")
+    if (B, S, h) == (20, 512, 16):  # 40 x 12 tiles of 256 x 256 beat 40 x 17 of 256 x 192: the widest tile's head split
+        assert name.value.decode() == "dma_agpr4w_256x256"
     ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), None, B * S, 3 * H, H, H, H, 3 * H, capi.EPI_QKV_SPLIT,
                             ctypes.byref(args), TTMI_DTYPES[dt], stream()))
     qkv = oracle.matmul(rounded(A, dt), rounded(W, dt), True)

@@ -419,10 +419,13 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     using BiasT = typename std::remove_cv<typename std::remove_pointer<decltype(bias)>::type>::type;
     const int m_lim = g.m, n_lim = tile_n < g.split_tiles ? g.split_col : g.n;  // a tile in front of the split ends there
     // bias of this lane's column groups, requested now so that it has landed when the epilogue wants it
-    // The epilogue works on groups of 32 rows; a lane contributes NV units of eight consecutive columns to each.
+    // The epilogue works on groups of GROUP rows; a lane contributes NV units of eight consecutive columns to each.
     // MF = 32: unit v = (block column v/2, half v%2 of its 32 columns), the lane's row is lrow.  MF = 16: unit v =
-    // (16-row block v / (CB/2) of the pair, pair of block columns v % (CB/2)), the lane's row is 16*(v / (CB/2)) + lrow.
-    constexpr int NV = MF == 32 ? CB * 2 : CB;
+    // (16-row block v / (CB/2) of the group, pair of block columns v % (CB/2)), the lane's row is 16*(v / (CB/2)) + lrow.
+    // (the widest tile of the 16-wide blocks stages 16 rows at a time: half the registers for the staged pieces, which
+    // its head-split epilogue does not have to spare)
+    constexpr int GROUP = (MF == 16 && BN > 192) ? 16 : 32;
+    constexpr int NV = MF == 32 ? CB * 2 : (GROUP == 32 ? CB : CB / 2);
     constexpr int NBV = MF == 32 ? NV : CB / 2;  // distinct column groups among the units (= bias vectors to hold)
     auto unit_chunk = [&](int v) __attribute__((always_inline)) {  // which group of eight columns of the wavefront's BN/2
       if constexpr (MF == 32) return (v / 2) * 4 + (v % 2) * 2 + lgrp;
@@ -453,7 +456,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       // bytes per lane.  A lone wavefront on a SIMD hides no latency by itself, so the order is written out: the
       // arithmetic of row block i runs while the strip reads of block i-1 are in flight, then the stores of block
       // i-1 go out back to back, then block i is written to the strip and its reads are issued.
-      constexpr int GROUP = 32, GROUPS = 128 / GROUP;  // rows staged at a time
+      constexpr int GROUPS = 128 / GROUP;
       constexpr int PASSES = GROUP * CPR / kWave;
       static_assert(GROUP * CPR % kWave == 0, "whole passes over a strip");
       int rd_off[PASSES], st_row[PASSES], st_col[PASSES], wr_off[NV];
@@ -506,8 +509,8 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
                 a = acc_read(acc[i][v / 2][8 * (v % 2) + e]);
                 b = acc_read(acc[i][v / 2][8 * (v % 2) + 4 + e]);
               } else {
-                a = acc_read(acc[2 * i + v / (CB / 2)][2 * (v % (CB / 2))][e]);
-                b = acc_read(acc[2 * i + v / (CB / 2)][2 * (v % (CB / 2)) + 1][e]);
+                a = acc_read(acc[(GROUP / 16) * i + v / (CB / 2)][2 * (v % (CB / 2))][e]);
+                b = acc_read(acc[(GROUP / 16) * i + v / (CB / 2)][2 * (v % (CB / 2)) + 1][e]);
               }
               pair_swap<MF>(a, b);
               out[e] = a;
@@ -742,16 +745,30 @@ struct LargeTileKernel<T, EpiQkvSplit<T, false>, typename std::enable_if<sizeof(
   static bool split_run(const GemmArgs& g, const Epi& epi) {
     return epi.v_pitch > 0 && g.n == 3 * epi.hidden && (2 * epi.hidden) % 192 != 0;
   }
+  // cost of the 192-wide tiles with the tile columns the two runs really have (one or two of them ragged)
+  static double cost192(const GemmArgs& g, const Epi& epi, int batch) {
+    const int64_t columns = split_run(g, epi) ? ceil_div(2 * epi.hidden, 192) + ceil_div(epi.hidden, 192) : ceil_div(g.n, 192);
+    return tile_cost(kW4Tile192, g.m, columns * 192, batch);
+  }
+  // the 256-wide tile serves widths it divides, V third included; its head-split epilogue spills some registers, so
+  // it is rated a little below the 256-wide tile of the row-major epilogues
+  static constexpr TileConfig kTile256{256, 256, 1, 1.07f};
+  static bool fits256(const GemmArgs& g, const Epi& epi) { return g.n % 256 == 0 && (epi.v_pitch == 0 || (2 * epi.hidden) % 256 == 0); }
+  static double cost(const GemmArgs& g, const Epi& epi, int batch) {
+    return std::min(cost192(g, epi, batch), fits256(g, epi) ? tile_cost(kTile256, g.m, g.n, batch) : 1e300);
+  }
   static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
-    if (!w4_wanted<T>(g, epi, batch, aligned)) return false;
-    if (!split_run(g, epi) || std::getenv("TTMI_LARGE_TILE") != nullptr) return true;
-    // the cost model again, with the tile columns the two runs really have (one or two of them ragged)
-    const int64_t columns = ceil_div(2 * epi.hidden, 192) + ceil_div(epi.hidden, 192);
+    if (!epi.vec || !w4_eligible<T>(g, batch, aligned)) return false;
+    if (const char* force = std::getenv("TTMI_LARGE_TILE")) {
+      if (force[0] == '0') return false;
+      if (force[0] == '1') return true;
+    }
     double other = 0;
     (void)pick_tile(g.m, g.n, batch, &other);
-    return tile_cost(kW4Tile192, g.m, columns * 192, batch) < other;
+    return cost(g, epi, batch) < other;
   }
   static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) {
+    if (fits256(g, epi) && tile_cost(kTile256, g.m, g.n, 1) < cost192(g, epi, 1)) return launch_w4<T, 256>(g, epi, s);
     return launch_w4<T, 192>(g, epi, s, split_run(g, epi) ? 2 * epi.hidden : 0);
   }
 };

@@ -24,6 +24,8 @@
 // feeds to MFMA kk.  No cross-lane shuffles of P, no LDS round trip for P.
 // exp() is evaluated as exp2; the mask (divided by the scale) seeds the score accumulators and
 // scale*log2(e) is applied inside the exp2 argument, so no separate scale/mask pass exists.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace ttmi {
@@ -358,8 +360,21 @@ int ttmi_fused_attention(const void* q, const void* k, const void* v, const floa
   uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                    reinterpret_cast<uintptr_t>(out);
   TTMI_REQUIRE((bits & 15) == 0, "tensors must be 16-byte aligned");
-  // eight wavefronts (256 queries) per workgroup once a sequence is longer than the 128 queries four of them cover
-  const int nw = seq > 128 ? 8 : 4;
+  // Eight wavefronts (256 queries) per workgroup when the sequence is longer than the 128 queries four of them cover
+  // AND the four-wavefront workgroups would already fill the chip (four of them fit a CU): a smaller problem runs
+  // faster on more, smaller workgroups.
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  int nw = (seq > 128 && ceil_div(seq, 128) * batch * heads >= 4 * (int64_t)cus) ? 8 : 4;
+  // TTMI_ATTENTION_WAVES=4 / 8 overrides the choice (A/B timing, and tests of the eight-wavefront form on small shapes)
+  if (const char* force = std::getenv("TTMI_ATTENTION_WAVES")) {
+    if (force[0] == '4') nw = 4;
+    if (force[0] == '8') nw = 8;
+  }
   const dim3 grid((unsigned)ceil_div(seq, nw * 32), (unsigned)(batch * heads));
   const float sl2 = scale * 1.4426950408889634f, inv_scale = 1.0f / scale;
   hipStream_t s = (hipStream_t)stream;

@@ -238,3 +238,24 @@ def test_gemm_describe_names_the_variant_without_a_device():
         capi.check(lib.ttmi_gemm_describe(m, n, k, epi, ctypes.byref(args), capi.F16, buf, 64))
         assert re.fullmatch(r"(reg|dma|dma_agpr)\d+w_\d+x\d+(_splitk\d+)?", buf.value.decode()), buf.value
     assert lib.ttmi_gemm_describe(128, 768, 3072, capi.EPI_NONE, None, capi.F16, buf, 4) != 0  # too small for the answer
+
+
+def test_one_short_sequence_splits_k_only_where_a_second_launch_pays():
+    """128 tokens: the output projection and the second FFN product (24 tiles of 64 x 64) are cut along K; the
+    intermediate Linear (96 tiles) keeps bias + GELU in the GEMM in 16-bit types, where the reduction kernel's launch
+    costs more than the split saves, and is cut in fp32, where it does not."""
+    import ctypes
+    lib = capi.load()
+    buf = ctypes.create_string_buffer(64)
+    args = capi.EpilogueArgs()
+    args.act = capi.ACT_GELU
+
+    def variant(m, n, k, epi, dt):
+        capi.check(lib.ttmi_gemm_describe(m, n, k, epi, ctypes.byref(args), dt, buf, 64))
+        return buf.value.decode()
+
+    assert "_splitk" in variant(128, 768, 768, capi.EPI_NONE, capi.F16)
+    assert "_splitk" in variant(128, 768, 3072, capi.EPI_NONE, capi.F16)
+    assert variant(128, 3072, 768, capi.EPI_BIAS_ACT, capi.F16) == "reg4w_64x64"
+    assert variant(128, 3072, 768, capi.EPI_BIAS_ACT, capi.BF16) == "reg4w_64x64"
+    assert "_splitk" in variant(128, 3072, 768, capi.EPI_BIAS_ACT, capi.F32)

@@ -852,14 +852,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_layer_norm_kernel(const flo
 //     last valid row (their results are never stored).
 //   * MFMA operand fragments are double-buffered in registers: the LDS reads of k-substep
 //     kk+1 are issued before the MFMAs of kk.
-// LDS bytes of the fast kernel: two K-loop stages, or one stage plus the epilogue staging area
-// (which starts at the second stage and may run past it), whichever is larger.
+//   * the K loop runs over a ring of NS stages, NS - 1 K steps in flight while one is multiplied: two for the
+//     256-row tiles (a step is 0.5-1.3 us of matrix work), four for the 128 x 64 tile.
+// LDS bytes of the fast kernel: NS K-loop stages, or one stage plus the epilogue staging area
+// (which starts at the second stage and may run past the last), whichever is larger.
 template <int BM, int BN, int WM, int WN>
 constexpr int fast_epilogue_bytes() { return WM * WN * 32 * (BN / WN + 4) * 4; }
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int NS = 2>
 constexpr int fast_lds_bytes() {
   constexpr int stage = (BM + BN) * kRowBytes;
-  return stage + (fast_epilogue_bytes<BM, BN, WM, WN>() > stage ? fast_epilogue_bytes<BM, BN, WM, WN>() : stage);
+  constexpr int rest = (NS - 1) * stage;
+  return stage + (fast_epilogue_bytes<BM, BN, WM, WN>() > rest ? fast_epilogue_bytes<BM, BN, WM, WN>() : rest);
 }
 
 // Barrier that publishes DMA-filled LDS: every wavefront first waits for its own global->LDS loads
@@ -869,9 +872,19 @@ __device__ __forceinline__ void dma_landed_barrier() {
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
   __syncthreads();
 }
+// The same with the N youngest vector memory operations of the wavefront allowed to stay in flight (they complete
+// in order, so everything older has landed).  Written as instructions: __syncthreads() is a fence as well, and in
+// front of a fence the compiler waits for EVERY outstanding vector memory operation, the DMA loads of the later
+// stages included.  The wavefront's own LDS reads are waited for, so that the stage it has read may be refilled.
+template <int N>
+__device__ __forceinline__ void dma_landed_barrier_but() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a six-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
+}
 
-template <typename T, int BM, int BN, int WM, int WN, typename Epi>
+template <typename T, int BM, int BN, int WM, int WN, int NS, typename Epi>
 __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmArgs g, const Epi epi) {
+  static_assert(NS >= 2 && NS <= 4, "stages of the K-loop ring");
   constexpr int NW = WM * WN, NT = NW * kWave;
   constexpr int KPC = 16 / sizeof(T);
   constexpr int BK = kRowBytes / sizeof(T);
@@ -972,7 +985,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   // Software pipeline of one K step (4 k-substeps kk, TM*TN MFMAs each):
   //   kk = 0,1,2 : LDS reads of substep kk+1 interleaved with the MFMAs of kk
   //   wait for the DMA of the next stage + barrier   (everyone has also read all of this stage)
-  //   issue the DMA of step kt+2 into the stage just drained
+  //   issue the DMA of step kt+NS into the stage just drained
   //   kk = 3     : LDS reads of substep 0 of the NEXT stage interleaved with the MFMAs of kk = 3
   // so neither the LDS latency nor the barrier leaves the MFMA pipe without queued work.
   // sched_group_barrier pins the interleaving (mask 0x100 = LDS read, 0x008 = MFMA).
@@ -1014,13 +1027,16 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
     dma_landed_barrier();  // step 0 has landed; the previous tile's staging area has been read out
-    if (ksteps > 1) issue(1);
+#pragma unroll
+    for (int st = 1; st < NS; ++st)
+      if (st < ksteps) issue(st);
     Chunk fa[2][TM], fb[2][TN];
     read_frags(smem, 0, fa[0], fb[0]);
+    int cur = 0;
     for (int kt = 0; kt < ksteps; ++kt) {
-      const int cur = kt & 1;
+      const int nxt = cur + 1 == NS ? 0 : cur + 1;
       const char* st = smem + cur * STAGE;
-      const char* st_next = smem + (cur ^ 1) * STAGE;
+      const char* st_next = smem + nxt * STAGE;
       read_frags(st, 1, fa[1], fb[1]);
       mma_step(fa[0], fb[0]);
       interleave();
@@ -1030,11 +1046,22 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
       read_frags(st, 3, fa[1], fb[1]);
       mma_step(fa[0], fb[0]);
       interleave();
-      dma_landed_barrier();  // the other stage is complete, and everyone has read all of this one
-      if (kt + 2 < ksteps) issue(cur);
+      // step kt+1 is complete, and everyone has read all of this stage.  Steps kt+2 .. kt+NS-1 (those that
+      // exist) stay in flight: each is the youngest A_LOADS + B_LOADS operations of this wavefront.
+      if constexpr (NS == 2) {
+        dma_landed_barrier();
+      } else {
+        constexpr int LPS = A_LOADS + B_LOADS;
+        const int younger = min(kt + NS - 1, ksteps - 1) - (kt + 1);
+        if (NS >= 4 && younger >= 2) dma_landed_barrier_but<(NS >= 4 ? 2 : 0) * LPS>();
+        else if (younger >= 1) dma_landed_barrier_but<LPS>();
+        else dma_landed_barrier_but<0>();
+      }
+      if (kt + NS < ksteps) issue(cur);
       read_frags(st_next, 0, fa[0], fb[0]);  // harmless on the last step
       mma_step(fa[1], fb[1]);
       interleave();
+      cur = nxt;
     }
     __syncthreads();  // all LDS reads of this tile are done
 
@@ -1047,7 +1074,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
       // stores, one round trip per strip; after this wait the strips' stores are issued back to back.
       __builtin_amdgcn_s_waitcnt(0x0F70);
     }
-    store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN>() - STAGE>(acc, bj, smem + STAGE, epi, g, z_epi, m0 + wm0,
+    store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN, NS>() - STAGE>(acc, bj, smem + STAGE, epi, g, z_epi, m0 + wm0,
                                                                          n0 + wn0, lane, wave);
     if (next >= xcd_end) break;
     logical = next;
@@ -1111,10 +1138,10 @@ static int compute_units() {
   return cus;
 }
 
-template <typename T, int BM, int BN, int WM, int WN, typename Epi>
+template <typename T, int BM, int BN, int WM, int WN, typename Epi, int NS = 2>
 static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   constexpr int NT = WM * WN * kWave;
-  constexpr int LDS = fast_lds_bytes<BM, BN, WM, WN>();
+  constexpr int LDS = fast_lds_bytes<BM, BN, WM, WN, NS>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
   if (describe_only("dma", WM * WN, BM, BN)) return 0;
   g.tiles_m = (g.m + BM - 1) / BM;
@@ -1127,7 +1154,7 @@ static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
       tiles >= kXcdRemapMinTiles
           ? (unsigned)(std::min(ceil_div(tiles, kNumXcd), std::max<int64_t>(1, resident / kNumXcd)) * kNumXcd)
           : (unsigned)tiles;
-  auto kern = gemm_fast_kernel<T, BM, BN, WM, WN, Epi>;
+  auto kern = gemm_fast_kernel<T, BM, BN, WM, WN, NS, Epi>;
   if (LDS > 64 * 1024) {
     const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
     if (rc != 0) return rc;
@@ -1241,7 +1268,7 @@ static int launch_fast_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hi
   const bool vec = g.n % 4 == 0;
   EpiPartial part{ws, (int64_t)g.m * g.n, g.n, vec};
   constexpr int LDS = fast_lds_bytes<128, 128, 2, 2>();
-  auto kern = gemm_fast_kernel<T, 128, 128, 2, 2, EpiPartial>;
+  auto kern = gemm_fast_kernel<T, 128, 128, 2, 2, 2, EpiPartial>;
   {
     const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
     if (rc != 0) return rc;
@@ -1355,6 +1382,10 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
             if (plan.kind == SplitKind::kDmaTiles)
               return launch_fast_splitk<T>(g, plan.splits, g.k / BK, BK, s, ReduceWithEpilogue<Epi>{epi, g.m, g.n});
           }
+          // 128 x 128 tiles on at most half the CUs and a K too short to cut: 128 x 64 tiles put twice as many CUs
+          // to work (2560 x 768 x 768: 240 tiles in one round, 9 us against 11)
+          if (batch == 1 && tiles(128, 128) <= compute_units() / 2 && tiles(128, 64) <= compute_units())
+            return launch_fast<T, 128, 64, 2, 2, Epi, 4>(g, epi, batch, s);
           return launch_fast<T, 128, 128, 2, 2, Epi>(g, epi, batch, s);
         }
         // small problems are latency-bound: the register-staged kernel hides the global latency

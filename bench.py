@@ -13,6 +13,7 @@ the 20-request variable-length batch), the roofline of the dominant kernel measu
 HIP events, and the CPU oracle timed on the host cores of the same box.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
+    python bench.py --only-extra smart_batch|albert_f16_b8_s256|base_int8_b20_s128   (one other configuration, for profiling)
 """
 import argparse
 import ctypes
@@ -408,6 +409,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the other shapes of the metric")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline pass")
+    ap.add_argument("--only-extra", default=None, choices=["smart_batch", "albert_f16_b8_s256", "base_int8_b20_s128"],
+                    help="profiling helper: run just this other configuration of the metric, print its figures, exit")
     ap.add_argument("--pmc-kernel", default=None,
                     help="counter-collection helper: run one calibration copy and a few launches of the named kernel "
                          "of the roofline pass (e.g. ffn1_gemm+bias+gelu), print nothing, exit")
@@ -424,6 +427,12 @@ def main():
     layers, hidden, heads, ffn, dtype, batch, seq = WORKLOADS[args.workload]
     if args.pmc_kernel:
         kernel_rooflines(dtype, batch, seq, hidden, heads, ffn, iters=3, only=args.pmc_kernel)
+        return
+    if args.only_extra:
+        run = {"smart_batch": lambda: run_smart_batch(max(10, args.steps // 2), args.warmup),
+               "albert_f16_b8_s256": lambda: run_albert(args.steps, args.warmup),
+               "base_int8_b20_s128": lambda: run_int8(args.steps, args.warmup)}[args.only_extra]
+        print(json.dumps({args.only_extra: run()}))
         return
     head = run_dense(args.workload, args.steps, args.warmup)
     line = {

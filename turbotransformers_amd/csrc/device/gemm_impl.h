@@ -1351,7 +1351,9 @@ static SplitPlan plan_split(int64_t m, int64_t n, int64_t k, int64_t batch, bool
   if (tile == 3) {
     const int64_t t128 = ceil_div(m, 128) * ceil_div(n, 128);
     if (t128 <= compute_units() / 2 && ksteps >= 16) {
-      const int splits = (int)std::min<int64_t>({2 * (int64_t)compute_units() / t128, ksteps / 8, 8});
+      // one and a half workgroups per CU: with two (four slices at 2560 x 768, five at 2048 x 768) the extra fp32
+      // partial tiles cost more than the shorter K loops save (20 x 128 tokens -1.3 %, ALBERT 8 x 256 -3.3 % with one slice less)
+      const int splits = (int)std::min<int64_t>({3 * (int64_t)compute_units() / (2 * t128), ksteps / 8, 8});
       if (splits > 1) return {SplitKind::kDmaTiles, splits};
     }
   } else if (tile == 4) {

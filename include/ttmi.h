@@ -325,7 +325,8 @@ TTMI_API int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, i
 
 /* Which kernel variant ttmi_gemm (epilogue TTMI_EPI_NONE, args NULL) or ttmi_gemm_fused would launch for an
  * aligned, densely packed product of this shape, as text: family (reg = register-staged, dma = global->LDS DMA,
- * dma_agpr = DMA with accumulators in AGPRs), wavefronts per workgroup, tile, K split; e.g. "dma8w_256x256".
+ * dma_agpr = DMA with accumulators in AGPRs, wave = one wavefront per tile with its operand fragments straight from
+ * global memory), wavefronts per workgroup, tile, K split; e.g. "dma8w_256x256", "wave1w_32x32_splitk3".
  * Nothing is launched.  No counterpart in the reference (cuBLAS picks its kernels out of sight); measurement
  * scripts use it to tie recorded per-kernel figures to the variant they were recorded on.  For the QKV epilogues
  * `args` supplies seq / heads / head_dim / v_seq_pitch (and batch); pointers in it are ignored. */

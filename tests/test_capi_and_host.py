@@ -236,7 +236,7 @@ def test_gemm_describe_names_the_variant_without_a_device():
     for m, n, k, epi in [(32768, 3072, 768, capi.EPI_BIAS_ACT), (32768, 768, 3072, capi.EPI_NONE), (128, 768, 3072, capi.EPI_NONE),
                          (2560, 768, 3072, capi.EPI_BIAS)]:
         capi.check(lib.ttmi_gemm_describe(m, n, k, epi, ctypes.byref(args), capi.F16, buf, 64))
-        assert re.fullmatch(r"(reg|dma|dma_agpr)\d+w_\d+x\d+(_splitk\d+)?", buf.value.decode()), buf.value
+        assert re.fullmatch(r"(reg|dma|dma_agpr|wave)\d+w_\d+x\d+(_splitk\d+)?", buf.value.decode()), buf.value
     assert lib.ttmi_gemm_describe(128, 768, 3072, capi.EPI_NONE, None, capi.F16, buf, 4) != 0  # too small for the answer
 
 
@@ -256,6 +256,26 @@ def test_one_short_sequence_splits_k_only_where_a_second_launch_pays():
 
     assert "_splitk" in variant(128, 768, 768, capi.EPI_NONE, capi.F16)
     assert "_splitk" in variant(128, 768, 3072, capi.EPI_NONE, capi.F16)
-    assert variant(128, 3072, 768, capi.EPI_BIAS_ACT, capi.F16) == "reg4w_64x64"
-    assert variant(128, 3072, 768, capi.EPI_BIAS_ACT, capi.BF16) == "reg4w_64x64"
+    assert variant(128, 3072, 768, capi.EPI_BIAS_ACT, capi.F16) == "wave1w_32x32"
+    assert variant(128, 3072, 768, capi.EPI_BIAS_ACT, capi.BF16) == "wave1w_32x32"
     assert "_splitk" in variant(128, 3072, 768, capi.EPI_BIAS_ACT, capi.F32)
+
+
+def test_up_to_128_rows_of_16_bit_operands_take_the_wavefront_kernel():
+    """One wavefront per 32 x 32 tile, operand fragments straight from global memory: 16-bit types, at most 128 rows,
+    K a multiple of the 128-byte step; fp32 and longer inputs stay on the LDS-tiled kernels."""
+    import ctypes
+    lib = capi.load()
+    buf = ctypes.create_string_buffer(64)
+
+    def variant(m, n, k, dt):
+        capi.check(lib.ttmi_gemm_describe(m, n, k, capi.EPI_NONE, None, dt, buf, 64))
+        return buf.value.decode()
+
+    for m in (1, 10, 40, 128):
+        assert variant(m, 2304, 768, capi.F16).startswith("wave1w_32x32")  # cut along K while its tiles are few
+        assert variant(m, 2304, 768, capi.BF16).startswith("wave1w_32x32")
+        assert variant(m, 768, 3072, capi.F16).startswith("wave1w_32x32_splitk")
+    assert not variant(128, 2304, 768, capi.F32).startswith("wave")
+    assert not variant(129, 2304, 768, capi.F16).startswith("wave")
+    assert not variant(128, 2304, 776, capi.F16).startswith("wave")

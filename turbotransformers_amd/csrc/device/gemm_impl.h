@@ -716,6 +716,74 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
   store_tile<T, TM, TN, NT, 2 * STAGE>(acc, bj, smem, epi, g, z_epi, m0 + wm0, n0 + wn0, lane, wave);
 }
 
+// ------------------------------------------------------------------ wavefront kernel -----
+// For a handful of rows (one short sequence: M <= 128) the product is a chain of short launches, and what a launch
+// costs beyond its fixed 4 us is the bytes its busiest CU has to fetch and the barriers of its K loop.  Here a
+// workgroup is ONE wavefront that owns a 32 x 32 tile: its MFMA operand fragments are 16 contiguous bytes of a row
+// of A and of W, so every lane fetches its fragments straight from global memory into registers (no LDS, no
+// barrier, DEPTH K steps of eight loads in flight), and a 128 x 2304 x 768 product is 288 wavefronts over all CUs
+// instead of 72 workgroups over 72.  Tiles walk column by column (the four row tiles of a weight panel are
+// neighbours and share it in one XCD's L2).  16-bit types, W as [N,K], K a multiple of the 128-byte step.
+template <typename T, int DEPTH, typename Epi>
+__global__ __launch_bounds__(kWave) void gemm_wave_kernel(const GemmArgs g, const Epi epi) {
+  static_assert(sizeof(T) == 2, "16-bit operands");
+  constexpr int BK = kRowBytes / sizeof(T);  // 64 elements per K step, four MFMAs
+  using Acc = typename Mma<T>::Acc;
+  constexpr int STRIP = 32 * (32 + 4) * 4;   // store_tile's staging strip of one wavefront
+  __shared__ __align__(16) char strip[STRIP];
+
+  const int tiles = g.tiles_m * g.tiles_n;
+  const bool remap = tiles >= kXcdRemapMinTiles;
+  const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
+  const int logical = remap ? (int)(blockIdx.x % kNumXcd) * per_xcd + (int)(blockIdx.x / kNumXcd) : (int)blockIdx.x;
+  if (logical >= tiles) return;
+  int tile_m, tile_n;
+  tile_coords(logical, g.tiles_m, g.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * 32, n0 = tile_n * 32;
+  const int lane = threadIdx.x, lrow = lane & 31, lhalf = lane >> 5;
+
+  int kdim = g.k, k_lo = 0, z_epi = 0;
+  if (g.k_chunk > 0) {  // split-K: this wavefront sums a slice of K into its own partial tile
+    k_lo = (int)blockIdx.y * g.k_chunk;
+    kdim = min(g.k_chunk, g.k - k_lo);
+    z_epi = (int)blockIdx.y;
+  }
+  // rows past the edge are clamped to the last one: their results are never stored
+  const T* pa = reinterpret_cast<const T*>(g.a) + (int64_t)min(m0 + lrow, g.m - 1) * g.lda + k_lo + lhalf * 8;
+  const T* pb = reinterpret_cast<const T*>(g.b) + (int64_t)min(n0 + lrow, g.n - 1) * g.ldb + k_lo + lhalf * 8;
+
+  float bj[1];
+  load_bias_columns<1>(epi, n0 + lrow, g.n, bj);
+  Acc acc[1][1];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[0][0][e] = 0;
+
+  const int ksteps = kdim / BK;
+  Chunk ra[DEPTH][4], rb[DEPTH][4];
+  auto fetch = [&](int kt, Chunk (&a)[4], Chunk (&b)[4]) __attribute__((always_inline)) {
+    if (kt < ksteps) {
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        a[kk] = *reinterpret_cast<const Chunk*>(pa + kt * BK + kk * 16);
+        b[kk] = *reinterpret_cast<const Chunk*>(pb + kt * BK + kk * 16);
+      }
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) fetch(d, ra[d], rb[d]);
+  for (int kt0 = 0; kt0 < ksteps; kt0 += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      if (kt0 + u < ksteps) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) Mma<T>::run(ra[u][kk], rb[u][kk], acc[0][0]);
+        fetch(kt0 + u + DEPTH, ra[u], rb[u]);
+      }
+    }
+  }
+  store_tile<T, 1, 1, kWave, STRIP>(acc, bj, strip, epi, g, z_epi, m0, n0, lane, 0);
+}
+
 // ---------------------------------------------------------------------------- split-K -----
 // Few output tiles and a long K (one short sequence through the FFN: 24 tiles, 48..96 K steps)
 // leave most of the chip idle behind a long serial chain.  Then K is cut into `splits` slices,
@@ -1224,10 +1292,43 @@ static int pick_splits(int64_t m, int64_t n, int64_t ksteps, int64_t batch, size
   return (int)std::max<int64_t>(1, std::min<int64_t>({(int64_t)compute_units() / tiles, ksteps / 4, 16}));
 }
 
+// The wavefront kernel takes 16-bit problems of at most 128 rows on the [N,K] path (TTMI_WAVE_KERNEL=0 keeps them on
+// the 64 x 64 tiles, for A/B timing).
+constexpr int kWaveDepth = 4;  // K steps a wavefront keeps in flight: 32 loads of 16 bytes per lane
+template <typename T>
+static bool wave_kernel_ok(const GemmArgs& g, int batch, bool aligned) {
+  if (sizeof(T) != 2 || !aligned || batch != 1 || g.m > 128 || g.k % (kRowBytes / (int)sizeof(T)) != 0) return false;
+  if (const char* sw = getenv("TTMI_WAVE_KERNEL")) return sw[0] != '0';
+  return true;
+}
+// K slices for it: up to two wavefronts per CU, at least four K steps per slice.
+static int wave_splits(int64_t m, int64_t n, int64_t ksteps) {
+  const int64_t tiles = ceil_div(m, 32) * ceil_div(n, 32);
+  return (int)std::max<int64_t>(1, std::min<int64_t>({2 * (int64_t)compute_units() / tiles, ksteps / 4, 16}));
+}
+static void wave_grid(GemmArgs& g, unsigned* grid_x) {
+  g.tiles_m = (g.m + 31) / 32;
+  g.tiles_n = (g.n + 31) / 32;
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  *grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
+}
+template <typename T, typename Epi>
+static int launch_wave(GemmArgs g, const Epi& epi, hipStream_t s) {
+  if constexpr (sizeof(T) == 2) {
+    if (describe_only("wave", 1, 32, 32)) return 0;
+    unsigned grid_x = 0;
+    wave_grid(g, &grid_x);
+    hipLaunchKernelGGL((gemm_wave_kernel<T, kWaveDepth, Epi>), dim3(grid_x, 1, 1), dim3(kWave), 0, s, g, epi);
+  }
+  return launch_status("gemm_wave_kernel");
+}
+
 // `reduce(ws, slices, vec, stream)` launches the kernel that sums the slices and applies the epilogue.
 template <typename T, typename Reduce>
 static int launch_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStream_t s, const Reduce& reduce) {
-  if (describe_only("reg", 4, 64, 64, splits)) return 0;
+  const bool wave = wave_kernel_ok<T>(g, 1, true);  // callers come here with aligned operands and one problem
+  if (wave) splits = std::max(2, wave_splits(g.m, g.n, ksteps));
+  if (describe_only(wave ? "wave" : "reg", wave ? 1 : 4, wave ? 32 : 64, wave ? 32 : 64, splits)) return 0;
   const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
   float* ws = nullptr;
   {
@@ -1236,11 +1337,20 @@ static int launch_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStre
   }
   g.k_chunk = (int)ceil_div(ksteps, splits) * bk;
   const int used = (int)ceil_div(g.k, g.k_chunk);  // slices that actually hold part of K
+  const bool vec = g.n % 4 == 0;
+  EpiPartial part{ws, (int64_t)g.m * g.n, g.n, vec};
+  if constexpr (sizeof(T) == 2) {
+    if (wave) {
+      unsigned wgrid = 0;
+      wave_grid(g, &wgrid);
+      hipLaunchKernelGGL((gemm_wave_kernel<T, kWaveDepth, EpiPartial>), dim3(wgrid, (unsigned)used, 1), dim3(kWave), 0, s, g, part);
+      reduce(ws, used, vec, s);
+      return launch_status("gemm_wave_splitk");
+    }
+  }
   g.tiles_m = (g.m + 63) / 64;
   g.tiles_n = (g.n + 63) / 64;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-  const bool vec = g.n % 4 == 0;
-  EpiPartial part{ws, (int64_t)g.m * g.n, g.n, vec};
   constexpr int LDS = 2 * (64 + 64) * kRowBytes;
   const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
   hipLaunchKernelGGL((gemm_kernel<T, 64, 64, 2, 2, false, true, 2, EpiPartial>), dim3(grid_x, (unsigned)used, 1), dim3(256), LDS, s,
@@ -1397,6 +1507,7 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
             const SplitPlan plan = column_pass ? SplitPlan{SplitKind::kNone, 1} : plan_split<T>(g.m, g.n, g.k, batch, aligned);
             if (plan.kind == SplitKind::kSmallTiles)
               return launch_splitk<T>(g, plan.splits, g.k / BK, BK, s, ReduceWithEpilogue<Epi>{epi, g.m, g.n});
+            if (wave_kernel_ok<T>(g, batch, aligned)) return launch_wave<T>(g, epi, s);
           }
           return launch_config<T, 64, 64, 2, 2, false, true, Epi>(g, epi, batch, s);
         }

@@ -146,11 +146,12 @@ def test_large_tile_kernel_against_oracle_and_small_tiles(ttmi, oracle, large_ti
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
 @pytest.mark.parametrize("v_transposed", [False, True])
 @pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 100, 6, 64), (2, 300, 16, 64), (64, 32, 12, 64),
-                                     (20, 512, 16, 64)])
+                                     (20, 512, 16, 64), (7, 75, 12, 64), (6, 100, 12, 64)])
 def test_large_tile_kernel_qkv_split(ttmi, oracle, large_tile_forced, dt, B, S, h, d, v_transposed):
     """The same kernel behind the QKV projection: bias + head split, V row-major or transposed (those tiles run with
     the matrix operands unswapped and leave through the strip column-wise).  Sequence lengths that are and are not
-    multiples of 8 and of 32 (eight rows of one V^T store, the 32 rows of a staged group, may straddle two sequences),
+    multiples of 8 and of 32 (eight rows of one V^T store, the 32 rows of a staged group, may straddle two sequences;
+    a group of eight positions inside a sequence of a length off the 8-grid is one element-aligned 16-byte store),
     hidden sizes whose V third does and does not start on a multiple of the tile width (then the tile in front of it
     is cut short and a new run of tiles starts there)."""
     import ctypes
@@ -346,7 +347,8 @@ def test_fused_bias_and_bias_residual(ttmi, oracle, dt):
 
 @pytest.mark.parametrize("dt", ALL_DTYPES)
 @pytest.mark.parametrize("v_transposed", [False, True])
-@pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 7, 2, 32), (2, 300, 16, 64), (5, 13, 3, 64)])
+@pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 7, 2, 32), (2, 300, 16, 64), (5, 13, 3, 64),
+                                     (20, 100, 12, 64), (6, 60, 12, 64), (4, 27, 2, 64)])  # the last three: lengths off the 8-grid
 def test_fused_qkv_split(ttmi, oracle, dt, B, S, h, d, v_transposed):
     """QKV GEMM + SplitAddBiasTransposeForScore; with v_seq_pitch the V third lands transposed,
     [B,h,d,pitch] (pad columns untouched), everything else as before."""

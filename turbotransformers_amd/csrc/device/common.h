@@ -57,6 +57,17 @@ template <typename T, int N>
 __device__ __forceinline__ void store_vec(T* p, const Vec<T, N>& x) {
   *reinterpret_cast<Vec<T, N>*>(p) = x;
 }
+// The same store to an address that is only aligned to the element: global memory takes vector stores at any
+// alignment (the target's unaligned access mode, which the compiler relies on as well), so this is still one
+// instruction; a store that straddles a cache line costs a second request, nothing more.
+template <typename T, int N>
+struct __attribute__((packed, aligned(alignof(T)))) UnalignedVec {
+  Vec<T, N> x;
+};
+template <typename T, int N>
+__device__ __forceinline__ void store_vec_unaligned(T* p, const Vec<T, N>& x) {
+  reinterpret_cast<UnalignedVec<T, N>*>(p)->x = x;
+}
 
 // ---- wave64 reductions over groups of G lanes (G power of two <= 64) -------------------
 template <int G>

@@ -168,6 +168,25 @@ __device__ __forceinline__ void store_row8(T* p, const float (&v)[8]) {
 }
 
 template <typename T>
+__device__ __forceinline__ void store_row8_unaligned(T* p, const float (&v)[8]) {  // p aligned to the element only
+  if constexpr (sizeof(T) == 2) {
+    Vec<T, 8> o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o.v[j] = from_float<T>(v[j]);
+    store_vec_unaligned<T, 8>(p, o);
+  } else {
+    Vec<T, 4> lo, hi;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      lo.v[j] = from_float<T>(v[j]);
+      hi.v[j] = from_float<T>(v[j + 4]);
+    }
+    store_vec_unaligned<T, 4>(p, lo);
+    store_vec_unaligned<T, 4>(p + 4, hi);
+  }
+}
+
+template <typename T>
 __device__ __forceinline__ void load_row8(const T* p, float (&v)[8]) {
   if constexpr (sizeof(T) == 2) {
     Vec<T, 8> x = load_vec<T, 8>(p);
@@ -289,7 +308,8 @@ struct EpiQkvSplit {
   __device__ __forceinline__ bool column_pass() const { return v_pitch > 0; }
   __device__ __forceinline__ int first_column_of_pass() const { return 2 * hidden; }
   // Rows m..m+7 of output column n (n in the V third): eight consecutive sequence positions of
-  // one V^T row when they belong to one sequence, one 16-byte store.
+  // one V^T row when they belong to one sequence, one 16-byte store.  A sequence length that is no multiple
+  // of 8 shifts the groups of the later sequences off the 16-byte grid: the store is aligned to the element only.
   __device__ __forceinline__ void store_col8(int m, int m_limit, int n, float (&val)[8]) const {
     const uint32_t rem = (uint32_t)(n - 2 * hidden);
     const uint32_t head = div_dim.div(rem);
@@ -297,10 +317,10 @@ struct EpiQkvSplit {
     const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;  // b*seq + s
     const uint32_t b = div_seq.div(prow);
     const uint32_t s = prow - b * seq;
-    bool fast = m + 8 <= m_limit && (s & 7u) == 0 && s + 8 <= (uint32_t)seq;
+    bool fast = m + 8 <= m_limit && s + 8 <= (uint32_t)seq;
     if (PAD && fast) fast = (uint32_t)token_rows[m + 7] == prow + 7;
     if (fast) {
-      store_row8<T>(v + (((int64_t)b * heads + head) * dim + i) * v_pitch + s, val);
+      store_row8_unaligned<T>(v + (((int64_t)b * heads + head) * dim + i) * v_pitch + s, val);
       return;
     }
     for (int j = 0; j < 8 && m + j < m_limit; ++j) {
@@ -345,6 +365,12 @@ struct EpiQkvSplit {
     const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;
     const uint32_t b = div_seq.div(prow);
     return (int64_t)b * hidden * v_pitch + (prow - b * seq);
+  }
+  __device__ __forceinline__ int64_t vt_row_part(int m, uint32_t& s) const {  // also returns the position in the sequence
+    const uint32_t prow = PAD ? (uint32_t)token_rows[m] : (uint32_t)m;
+    const uint32_t b = div_seq.div(prow);
+    s = prow - b * seq;
+    return (int64_t)b * hidden * v_pitch + s;
   }
   __device__ __forceinline__ float finish(float x) const { return x; }
   __device__ __forceinline__ T* dest8(int m, int n) const {  // head_dim % 8 == 0: the eight columns stay in one head
@@ -1458,7 +1484,13 @@ static SplitPlan plan_split(int64_t m, int64_t n, int64_t k, int64_t batch, bool
   if (!aligned || k % BK != 0 || batch != 1) return {SplitKind::kNone, 1};
   const int64_t ksteps = k / BK;
   const int tile = pick_tile(m, n, batch);
-  if (tile == 3) {
+  if (tile == 4) {
+    const int splits = pick_splits(m, n, ksteps, batch, sizeof(T));
+    if (splits > 1) return {SplitKind::kSmallTiles, splits};
+  }
+  // (the cost model knows nothing of K: a few hundred rows by 768 columns by K = 3072 are 150 tiles of 64 x 64, too many
+  // for the small split, each a serial chain of 48 K steps; cut on 128 x 128 tiles they are 250 workgroups of 8 steps)
+  if (tile == 3 || tile == 4) {
     const int64_t t128 = ceil_div(m, 128) * ceil_div(n, 128);
     if (t128 <= compute_units() / 2 && ksteps >= 16) {
       // one and a half workgroups per CU: with two (four slices at 2560 x 768, five at 2048 x 768) the extra fp32
@@ -1466,9 +1498,6 @@ static SplitPlan plan_split(int64_t m, int64_t n, int64_t k, int64_t batch, bool
       const int splits = (int)std::min<int64_t>({3 * (int64_t)compute_units() / (2 * t128), ksteps / 8, 8});
       if (splits > 1) return {SplitKind::kDmaTiles, splits};
     }
-  } else if (tile == 4) {
-    const int splits = pick_splits(m, n, ksteps, batch, sizeof(T));
-    if (splits > 1) return {SplitKind::kSmallTiles, splits};
   }
   return {SplitKind::kNone, 1};
 }
@@ -1507,6 +1536,8 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
             const SplitPlan plan = column_pass ? SplitPlan{SplitKind::kNone, 1} : plan_split<T>(g.m, g.n, g.k, batch, aligned);
             if (plan.kind == SplitKind::kSmallTiles)
               return launch_splitk<T>(g, plan.splits, g.k / BK, BK, s, ReduceWithEpilogue<Epi>{epi, g.m, g.n});
+            if (plan.kind == SplitKind::kDmaTiles)
+              return launch_fast_splitk<T>(g, plan.splits, g.k / BK, BK, s, ReduceWithEpilogue<Epi>{epi, g.m, g.n});
             if (wave_kernel_ok<T>(g, batch, aligned)) return launch_wave<T>(g, epi, s);
           }
           return launch_config<T, 64, 64, 2, 2, false, true, Epi>(g, epi, batch, s);

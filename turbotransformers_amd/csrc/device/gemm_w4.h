@@ -614,13 +614,19 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
           if (u > 0) {
             const int j = (u - 1) / 2, hf = (u - 1) % 2;
             const int m = m0 + wm0 + hf * 64 + rd_chunk * 8;
-            const int64_t row_off = epi.vt_row_part(min(m, m_lim - 1));
+            uint32_t seq_pos = 0;
+            const int64_t row_off = epi.vt_row_part(min(m, m_lim - 1), seq_pos);
+            // the eight rows are eight positions of one sequence: still one store, though off the 16-byte grid where
+            // the sequence length is no multiple of 8
+            const bool in_sequence = m + 8 <= m_lim && seq_pos + 8 <= (uint32_t)epi.seq;
 #pragma unroll
             for (int p = 0; p < VP; ++p) {
               const int ncol = n0 + wn0 + j * 32 + p * 8 + rd_col;
               T* dst = vt_base + (int64_t)(j * 32 + p * 8) * epi.v_pitch + row_off;
               if (rows_whole) {
                 if (ncol < n_lim) *reinterpret_cast<Quad*>(dst) = vt_landed[p];
+              } else if (in_sequence) {
+                if (ncol < n_lim) store_vec_unaligned<T, 8>(dst, __builtin_bit_cast(Vec<T, 8>, vt_landed[p]));
               } else if (m < m_lim && ncol < n_lim) {
                 const Vec<T, 8> x = __builtin_bit_cast(Vec<T, 8>, vt_landed[p]);
                 float out[8];

@@ -296,8 +296,9 @@ void MultiHeadedAttentionSmartBatch::operator()(const Tensor& key_tensor, const 
   // Padded q,k,v; the QKV GEMM scatters bias-added rows of the packed input into them.  The
   // unfused core multiplies whole padded tensors, so pad rows must be exactly 0 there
   // (transpose.cpp:504-522); the fused kernel never reads a pad row, so nothing is cleared.
-  // V stays row-major here: sequences start at arbitrary packed rows, so a transposed store could
-  // rarely use 16-byte vectors, and that costs the QKV GEMM more than the scatter costs the attention kernel.
+  // V stays row-major here: the transposed store needs the row map and a division per group of eight packed rows,
+  // and that costs the QKV GEMM more than the scatter costs the attention kernel (20 requests, 6275 tokens:
+  // 2.50 against 2.39 ms per forward).
   const bool fused_core = UseFusedCore(attention_mask, att_score, d, dt);
   Tensor* qkv[3] = {&q_, &k_, &v_};
   const char* names[3] = {"self/q/Reshape", "self/k/Reshape", "self/v/Reshape"};

@@ -279,3 +279,24 @@ def test_up_to_128_rows_of_16_bit_operands_take_the_wavefront_kernel():
     assert not variant(128, 2304, 768, capi.F32).startswith("wave")
     assert not variant(129, 2304, 768, capi.F16).startswith("wave")
     assert not variant(128, 2304, 776, capi.F16).startswith("wave")
+
+
+def test_transposed_v_of_sequences_shorter_than_8_stays_off_the_one_wavefront_per_simd_kernel():
+    """That kernel stores a group of eight rows of a transposed V that leaves its sequence element by element into
+    this sequence and the next one; with fewer than 8 positions per sequence a group would touch three, so such a
+    QKV projection runs on the other kernels however many rows it has."""
+    import ctypes
+    lib = capi.load()
+    buf = ctypes.create_string_buffer(64)
+
+    def variant(batch, seq, pitch):
+        args = capi.EpilogueArgs()
+        args.bias = args.q = args.k = args.v = 1 << 20  # never dereferenced: describe launches nothing
+        args.seq, args.heads, args.head_dim, args.v_seq_pitch = seq, 12, 64, pitch
+        capi.check(lib.ttmi_gemm_describe(batch * seq, 2304, 768, capi.EPI_QKV_SPLIT, ctypes.byref(args), capi.F16, buf, 64))
+        return buf.value.decode()
+
+    assert variant(1000, 12, 16).startswith("dma_agpr4w")
+    assert variant(1500, 8, 8).startswith("dma_agpr4w")
+    assert variant(2400, 5, 0).startswith("dma_agpr4w")  # row-major V: any length
+    assert not variant(2400, 5, 8).startswith("dma_agpr4w")

@@ -348,7 +348,7 @@ def test_fused_bias_and_bias_residual(ttmi, oracle, dt):
 @pytest.mark.parametrize("dt", ALL_DTYPES)
 @pytest.mark.parametrize("v_transposed", [False, True])
 @pytest.mark.parametrize("B,S,h,d", [(2, 40, 12, 64), (16, 128, 12, 64), (3, 7, 2, 32), (2, 300, 16, 64), (5, 13, 3, 64),
-                                     (20, 100, 12, 64), (6, 60, 12, 64), (4, 27, 2, 64)])  # the last three: lengths off the 8-grid
+                                     (20, 100, 12, 64), (6, 60, 12, 64), (4, 27, 2, 64), (300, 5, 12, 64)])  # the last four: lengths off the 8-grid
 def test_fused_qkv_split(ttmi, oracle, dt, B, S, h, d, v_transposed):
     """QKV GEMM + SplitAddBiasTransposeForScore; with v_seq_pitch the V third lands transposed,
     [B,h,d,pitch] (pad columns untouched), everything else as before."""

@@ -26,10 +26,13 @@ DEVICE_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-I", INCLUDE,
+    # A "#pragma unroll" the optimizer gives up on (the unrolled body grew past its size limit) leaves register
+    # arrays indexed at run time: slow, and wrong where accumulators are pinned by inline asm.  Fail the build instead.
+    "-Werror=pass-failed",
 ]
 # Per-file additions.  attention.hip: maxima over MFMA results would otherwise be preceded by one
 # canonicalising v_max per operand (signalling-NaN quieting), a tenth of the softmax's VALU work.
-DEVICE_FILE_FLAGS = {"attention.hip": ["-fno-honor-nans"]}
+DEVICE_FILE_FLAGS = {"attention.hip": ["-fno-honor-nans"], "gemm.hip": ["-mllvm", "-pragma-unroll-threshold=65536"]}
 
 
 def _run(cmd):

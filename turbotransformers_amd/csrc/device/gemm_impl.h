@@ -323,12 +323,25 @@ struct EpiQkvSplit {
       store_row8_unaligned<T>(v + (((int64_t)b * heads + head) * dim + i) * v_pitch + s, val);
       return;
     }
-    for (int j = 0; j < 8 && m + j < m_limit; ++j) {
+    // The group straddles two sequences (or the end of the matrix).  Unrolled with constant indices: a loop with a
+    // run-time trip count would index val[] dynamically and push it to scratch memory.
+    if (!PAD && seq >= 8) {  // the next sequence starts hidden * v_pitch elements further on
+      T* dst = v + (((int64_t)b * heads + head) * dim + i) * v_pitch + s;
+      const int64_t hop = vt_hop();
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (m + j < m_limit) dst[j + (s + j >= (uint32_t)seq ? hop : 0)] = from_float<T>(val[j]);
+      return;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (m + j >= m_limit) break;
       const uint32_t pr = PAD ? (uint32_t)token_rows[m + j] : (uint32_t)(m + j);
       const uint32_t bj = div_seq.div(pr);
       v[(((int64_t)bj * heads + head) * dim + i) * v_pitch + (pr - bj * seq)] = from_float<T>(val[j]);
     }
   }
+  __device__ __forceinline__ int64_t vt_hop() const { return (int64_t)hidden * v_pitch - seq; }
   __device__ __forceinline__ T* dest(uint32_t b, uint32_t s, uint32_t n) const {
     const uint32_t w = div_hidden.div(n);
     const uint32_t rem = n - w * hidden;

@@ -628,11 +628,16 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
               } else if (in_sequence) {
                 if (ncol < n_lim) store_vec_unaligned<T, 8>(dst, __builtin_bit_cast(Vec<T, 8>, vt_landed[p]));
               } else if (m < m_lim && ncol < n_lim) {
+                // the group runs over the end of its sequence into the next one, hidden * v_pitch elements further
+                // on (sequences of fewer than 8 positions off the 8-grid never come here, see wanted()), or over
+                // the end of the matrix: element by element, no division.  A rolled loop that picks its element
+                // with selects: unrolled, the epilogue grows past what the compiler unrolls of the loop over the
+                // units, and the accumulators would be indexed at run time.
                 const Vec<T, 8> x = __builtin_bit_cast(Vec<T, 8>, vt_landed[p]);
-                float out[8];
+                const int hop = (int)epi.vt_hop();
 #pragma unroll
-                for (int e = 0; e < 8; ++e) out[e] = to_float(x.v[e]);
-                epi.store_col8(m, m_lim, ncol, out);
+                for (int e = 0; e < 8; ++e)
+                  if (m + e < m_lim) dst[e + (seq_pos + e >= (uint32_t)epi.seq ? hop : 0)] = x.v[e];
               }
             }
           }
@@ -765,6 +770,8 @@ struct LargeTileKernel<T, EpiQkvSplit<T, false>, typename std::enable_if<sizeof(
   }
   static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
     if (!epi.vec || !w4_eligible<T>(g, batch, aligned)) return false;
+    // eight rows of a transposed V lie in at most two sequences: what the kernel's element-wise store assumes
+    if (epi.v_pitch > 0 && epi.seq < 8) return false;
     if (const char* force = std::getenv("TTMI_LARGE_TILE")) {
       if (force[0] == '0') return false;
       if (force[0] == '1') return true;

@@ -539,8 +539,8 @@ def _v_operand(V, dt, v_transposed, poison=True):
 
 @pytest.fixture(params=["auto", "8"])
 def attention_waves(request, monkeypatch):
-    """Wavefronts per workgroup of the fused attention kernel: its own choice (eight only for long sequences on a full
-    chip, which none of these small shapes is), and eight forced through TTMI_ATTENTION_WAVES."""
+    """Wavefronts per workgroup of the fused attention kernel: its own choice (eight only for long sequences with a workgroup
+    per compute unit, which none of these small shapes has), and eight forced through TTMI_ATTENTION_WAVES."""
     if request.param != "auto":
         monkeypatch.setenv("TTMI_ATTENTION_WAVES", request.param)
     return request.param

@@ -360,16 +360,19 @@ int ttmi_fused_attention(const void* q, const void* k, const void* v, const floa
   uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                    reinterpret_cast<uintptr_t>(out);
   TTMI_REQUIRE((bits & 15) == 0, "tensors must be 16-byte aligned");
-  // Eight wavefronts (256 queries) per workgroup when the sequence is longer than the 128 queries four of them cover
-  // AND the four-wavefront workgroups would already fill the chip (four of them fit a CU): a smaller problem runs
-  // faster on more, smaller workgroups.
+  // Eight wavefronts (256 queries) per workgroup stream the keys and values of their head once for twice the queries:
+  // a workgroup of that size costs about 1.6 times one of four wavefronts (20 x 136 tokens: 7.4 against 9.2 us;
+  // 64 x 512: 77 against 81).  Four win where the sequence fits them (up to 128 tokens), where two blocks of 256
+  // queries stand against three of 128 (257..384 tokens; 64 x 300: 44 against 49 us), and where even their workgroups
+  // are fewer than the compute units (4 x 512 tokens: 12.4 against 13.7 us).
   static const int cus = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
       n = 256;
     return n;
   }();
-  int nw = (seq > 128 && ceil_div(seq, 128) * batch * heads >= 4 * (int64_t)cus) ? 8 : 4;
+  const bool fits_four = seq <= 128 || 8 * ceil_div(seq, 256) >= 5 * ceil_div(seq, 128);
+  int nw = (fits_four || ceil_div(seq, 128) * batch * heads < (int64_t)cus) ? 4 : 8;
   // TTMI_ATTENTION_WAVES=4 / 8 overrides the choice (A/B timing, and tests of the eight-wavefront form on small shapes)
   if (const char* force = std::getenv("TTMI_ATTENTION_WAVES")) {
     if (force[0] == '4') nw = 4;

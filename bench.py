@@ -14,6 +14,7 @@ HIP events, and the CPU oracle timed on the host cores of the same box.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
     python bench.py --only-extra smart_batch|albert_f16_b8_s256|base_int8_b20_s128   (one other configuration, for profiling)
+    python bench.py --grid f16|bf16|f32   (the reference's fixed-length grid, this library beside PyTorch eager)
 """
 import argparse
 import ctypes
@@ -92,6 +93,27 @@ def run_dense(name, steps, warmup):
     return {"workload": name, "dtype": dtype, "batch": batch, "seq": seq, "ms_per_step": ms, "p50_ms": p50,
             "host_wall_ms_per_step": wall, "seq_per_s": batch / ms * 1e3,
             "tflops": (gemm + attn) / ms / 1e9, "frac_of_mfma_peak": (gemm + attn) / ms / 1e9 / PEAK_TFLOPS[dtype]}
+
+
+def run_grid(dtype, steps, warmup):
+    """The reference's fixed-length grid (benchmark/run_gpu_fixed_benchmark.sh:20-22: batch 1 and 20, 10 ... 500 tokens,
+    frameworks "turbo-transformers" and "torch"): ms per forward of this library and of the HuggingFace model run by
+    PyTorch itself (eager, its default scaled-dot-product attention) on the same GPU, same weights, same ids."""
+    import torch
+    tmodel, hf_model, cfg = build_model(12, 768, 12, 3072, dtype)
+    hf_model = hf_model.cuda()
+    g = torch.Generator().manual_seed(0)
+    rows = []
+    shapes = [(batch, seq) for batch in (1, 20) for seq in (10, 20, 40, 60, 80, 100, 200, 300, 400, 500)]
+    shapes.append((64, 512))  # not in the reference's grid: the shape the headline figure is quoted on
+    for batch, seq in shapes:
+        ids = torch.randint(0, cfg.vocab_size - 1, (batch, seq), generator=g, dtype=torch.int64).cuda()
+        ms, _, _, _ = time_steps(lambda: tmodel(ids), steps, warmup)
+        with torch.no_grad():
+            ms_torch, _, _, _ = time_steps(lambda: hf_model(ids), steps, warmup)
+        rows.append({"batch": batch, "seq": seq, "ms_per_step": ms, "pytorch_eager_ms_per_step": ms_torch,
+                     "speedup": ms_torch / ms})
+    return {"workload": "base_%s_fixed_length_grid" % dtype, "rows": rows}
 
 
 def run_smart_batch(steps, warmup):
@@ -411,6 +433,8 @@ def main():
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline pass")
     ap.add_argument("--only-extra", default=None, choices=["smart_batch", "albert_f16_b8_s256", "base_int8_b20_s128"],
                     help="profiling helper: run just this other configuration of the metric, print its figures, exit")
+    ap.add_argument("--grid", default=None, choices=["f16", "bf16", "f32"],
+                    help="time the reference's fixed-length grid (batch 1/20 x 10..500 tokens) beside PyTorch eager, print it as JSON and exit")
     ap.add_argument("--pmc-kernel", default=None,
                     help="counter-collection helper: run one calibration copy and a few launches of the named kernel "
                          "of the roofline pass (e.g. ffn1_gemm+bias+gelu), print nothing, exit")
@@ -427,6 +451,9 @@ def main():
     layers, hidden, heads, ffn, dtype, batch, seq = WORKLOADS[args.workload]
     if args.pmc_kernel:
         kernel_rooflines(dtype, batch, seq, hidden, heads, ffn, iters=3, only=args.pmc_kernel)
+        return
+    if args.grid:
+        print(json.dumps(run_grid(args.grid, args.steps, args.warmup)))
         return
     if args.only_extra:
         run = {"smart_batch": lambda: run_smart_batch(max(10, args.steps // 2), args.warmup),

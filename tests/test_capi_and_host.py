@@ -300,3 +300,23 @@ def test_transposed_v_of_sequences_shorter_than_8_stays_off_the_one_wavefront_pe
     assert variant(1500, 8, 8).startswith("dma_agpr4w")
     assert variant(2400, 5, 0).startswith("dma_agpr4w")  # row-major V: any length
     assert not variant(2400, 5, 8).startswith("dma_agpr4w")
+
+
+def test_fp32_products_pick_tiles_by_rounds_over_the_compute_units():
+    """fp32 is bound by the matrix pipe at every tile size, so the tile (and a cut along K) is chosen for whole
+    rounds of tiles over the CUs: a few thousand rows by 768 columns run on 64 x 64 tiles where the 16-bit types take
+    128 x 128, a last round that is nearly empty is filled by slices of K, large products keep the large tiles."""
+    import ctypes
+    lib = capi.load()
+    buf = ctypes.create_string_buffer(64)
+
+    def variant(m, n, k, dt):
+        capi.check(lib.ttmi_gemm_describe(m, n, k, capi.EPI_NONE, None, dt, buf, 64))
+        return buf.value.decode()
+
+    assert variant(4000, 768, 3072, capi.F32) == "reg4w_64x64"        # 756 tiles: three rounds of 256
+    assert variant(4000, 768, 3072, capi.F16) == "dma4w_128x128"
+    assert variant(1600, 768, 3072, capi.F32) == "reg4w_64x64_splitk5"  # 300 tiles are 1.17 rounds: 1500 slices, six
+    assert variant(1600, 768, 768, capi.F32) == "reg4w_64x64"          # K too short for the cut to pay
+    assert variant(32768, 3072, 768, capi.F32) == "dma8w_256x256"
+    assert variant(128, 768, 3072, capi.F32) == "reg4w_64x64_splitk10"  # one short sequence: as before

@@ -1463,11 +1463,22 @@ static double tile_cost(const TileConfig& c, int64_t m, int64_t n, int64_t batch
   return (double)full * c.per_cu * t + (double)ceil_div(rem, compute_units()) * t;
 }
 
-static int pick_tile(int64_t m, int64_t n, int64_t batch, double* cost_out = nullptr) {
+// fp32: the matrix pipe is sixteen times slower than for 16-bit operands and bounds every tile size, so what counts is
+// how evenly the tiles load the CUs (all wavefronts resident on a CU share its four SIMDs), and the small tiles lose
+// little: efficiencies fitted to a sweep of M = 800 ... 16384 by N, K = 768 / 3072 (4000 x 768 x 3072: 175 us on
+// 64 x 64 tiles, three per CU, against 233 us on 128 x 128, one on three CUs of four).
+constexpr float kTileEff32[] = {0.88f, 0.85f, 0.82f, 0.78f, 0.74f};
+static double tile_cost32(int i, int64_t m, int64_t n, int64_t batch) {
+  const TileConfig& c = kTileConfigs[i];
+  const int64_t tiles = ceil_div(m, c.bm) * ceil_div(n, c.bn) * batch;
+  return (double)ceil_div(tiles, compute_units()) * c.bm * c.bn / kTileEff32[i];
+}
+
+static int pick_tile(int64_t m, int64_t n, int64_t batch, double* cost_out = nullptr, size_t elem_size = 2) {
   int best = 0;
   double best_cost = 1e300;
   for (int i = 0; i < (int)(sizeof(kTileConfigs) / sizeof(kTileConfigs[0])); ++i) {
-    const double cost = tile_cost(kTileConfigs[i], m, n, batch);
+    const double cost = elem_size == 4 ? tile_cost32(i, m, n, batch) : tile_cost(kTileConfigs[i], m, n, batch);
     if (cost < best_cost) {
       best_cost = cost;
       best = i;
@@ -1496,14 +1507,35 @@ static SplitPlan plan_split(int64_t m, int64_t n, int64_t k, int64_t batch, bool
   constexpr int BK = kRowBytes / sizeof(T);
   if (!aligned || k % BK != 0 || batch != 1) return {SplitKind::kNone, 1};
   const int64_t ksteps = k / BK;
-  const int tile = pick_tile(m, n, batch);
+  const int tile = pick_tile(m, n, batch, nullptr, sizeof(T));
   if (tile == 4) {
     const int splits = pick_splits(m, n, ksteps, batch, sizeof(T));
     if (splits > 1) return {SplitKind::kSmallTiles, splits};
+    if (sizeof(T) == 4) {
+      // fp32 with more tiles than that: whole rounds of tiles over the CUs are what the launch costs, and a last round
+      // that is nearly empty (1600 x 768: 300 tiles, two rounds for 1.17 CUs' worth) is repaired by cutting K so that
+      // the slices fill the rounds.  Estimate in microseconds: matrix time of the rounds at the fitted efficiency plus
+      // the pass that sums the slices (their bytes at 4 TB/s and a launch); partial tiles of at most 32 MiB.
+      const int64_t tiles = ceil_div(m, 64) * ceil_div(n, 64);
+      const double per_round = 64.0 * 64.0 * 2.0 * (double)k / (157.3e6 / compute_units() * kTileEff32[4]);  // us, whole K
+      const double uncut = (double)ceil_div(tiles, compute_units()) * per_round;
+      double best = uncut;
+      int best_splits = 1;
+      for (int sp = 2; sp <= 8 && ksteps / sp >= 4 && (int64_t)sp * m * n * 4 <= (32ll << 20); ++sp) {
+        const double reduce = (double)(sp + 1) * m * n * 4 / 4e6 + 4.0;
+        const double t = (double)ceil_div(tiles * sp, compute_units()) * per_round / sp + reduce;
+        if (t < best) {
+          best = t;
+          best_splits = sp;
+        }
+      }
+      if (best < 0.9 * uncut) return {SplitKind::kSmallTiles, best_splits};
+    }
   }
   // (the cost model knows nothing of K: a few hundred rows by 768 columns by K = 3072 are 150 tiles of 64 x 64, too many
   // for the small split, each a serial chain of 48 K steps; cut on 128 x 128 tiles they are 250 workgroups of 8 steps)
-  if (tile == 3 || tile == 4) {
+  // (not fp32: there the 64 x 64 tiles the model picks for such a shape already load every SIMD)
+  if (sizeof(T) != 4 && (tile == 3 || tile == 4)) {
     const int64_t t128 = ceil_div(m, 128) * ceil_div(n, 128);
     if (t128 <= compute_units() / 2 && ksteps >= 16) {
       // one and a half workgroups per CU: with two (four slices at 2560 x 768, five at 2048 x 768) the extra fp32
@@ -1526,7 +1558,7 @@ static int launch_gemm(GemmArgs g, const Epi& epi, int batch, bool aligned, hipS
       bool column_pass = false;
       if constexpr (HasColumnPass<Epi>::value) column_pass = epi.v_pitch > 0;
       if (LargeTileKernel<T, Epi>::wanted(g, epi, batch, aligned)) return LargeTileKernel<T, Epi>::launch(g, epi, s);
-      switch (pick_tile(g.m, g.n, batch)) {
+      switch (pick_tile(g.m, g.n, batch, nullptr, sizeof(T))) {
         case 0: return launch_fast<T, 256, 256, 2, 4, Epi>(g, epi, batch, s);
         case 1: return launch_fast<T, 256, 192, 4, 2, Epi>(g, epi, batch, s);
         case 2: return launch_fast<T, 256, 128, 4, 2, Epi>(g, epi, batch, s);

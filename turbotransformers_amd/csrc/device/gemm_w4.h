@@ -771,7 +771,8 @@ struct LargeTileKernel<T, EpiQkvSplit<T, false>, typename std::enable_if<sizeof(
   static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
     if (!epi.vec || !w4_eligible<T>(g, batch, aligned)) return false;
     // eight rows of a transposed V lie in at most two sequences: what the kernel's element-wise store assumes
-    if (epi.v_pitch > 0 && epi.seq < 8) return false;
+    // (and steps from one sequence to the next with a 32-bit element offset)
+    if (epi.v_pitch > 0 && (epi.seq < 8 || (int64_t)epi.hidden * epi.v_pitch >= (1ll << 31))) return false;
     if (const char* force = std::getenv("TTMI_LARGE_TILE")) {
       if (force[0] == '0') return false;
       if (force[0] == '1') return true;

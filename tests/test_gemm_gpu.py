@@ -573,6 +573,34 @@ def test_fused_attention_vs_unfused_oracle(ttmi, oracle, attention_waves, dt, B,
     assert max_abs(host(out), want) <= GEMM_TOL[dt] * 2
 
 
+@pytest.mark.parametrize("B,h,S,masked", [(2, 3, 128, True), (1, 2, 512, False), (3, 2, 100, True), (2, 1, 37, True),
+                                         (1, 1, 500, True), (2, 12, 64, False), (1, 2, 1, False), (1, 1, 700, True),
+                                         (3, 2, 260, True), (2, 2, 63, False)])
+def test_fused_attention_fp32_vs_unfused_oracle(ttmi, oracle, attention_waves, B, h, S, masked):
+    """The fp32 form of the one-kernel attention (32x32x2 fp32 matrix instructions, V transposed with NaN in its pad
+    columns) against the oracle's four-step chain, to fp32 accuracy: nothing is rounded to 16 bits on the way."""
+    rng = np.random.default_rng(S + 3 * B)
+    d = 64
+    Q, K, V = (rng.standard_normal((B, h, S, d), np.float32) for _ in range(3))
+    mask = None
+    if masked:
+        mask = np.zeros((B, 1, 1, S), np.float32)
+        mask[0, ..., S // 2 + 1:] = -10000.0
+        mask[-1, ..., :S // 3] = -10000.0
+    dQ, dK = dev(Q, "f32"), dev(K, "f32")
+    dV, pitch = _v_operand(V, "f32", True)
+    out = torch.full((B, S, h * d), 9.0, dtype=torch.float32, device="cuda")
+    ok(ttmi.ttmi_fused_attention(ptr(dQ), ptr(dK), ptr(dV), ptr(dev(mask)) if masked else None, ptr(out), None, B, h, S, d,
+                                 pitch, 0.125, TTMI_DTYPES["f32"], stream()))
+    score = oracle.batch_matmul(Q, K, True, 0.125)
+    prob = oracle.apply_mask_and_softmax(score, mask, 1.0, True)
+    want = oracle.transpose_for_score(oracle.batch_matmul(prob, V, False)).reshape(B, S, h * d)
+    assert max_abs(host(out), want) <= 5e-5
+    # row-major V and packed batches are not built for fp32: refused, not miscomputed
+    assert ttmi.ttmi_fused_attention(ptr(dQ), ptr(dK), ptr(dev(V, "f32")), None, ptr(out), None, B, h, S, d, 0, 0.125,
+                                     TTMI_DTYPES["f32"], stream()) != 0
+
+
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
 @pytest.mark.parametrize("v_transposed", [False, True])
 @pytest.mark.parametrize("lens", [[70, 5, 129, 33], [300, 5, 257, 256]])

@@ -68,9 +68,9 @@ def test_bert_attention_vs_huggingface(tt, B, S):
     assert max_abs(host(got[0]), host(want[0])) < 1e-4  # bert_attention_test.py:92-96 (CPU bound)
     probs = torch.utils.dlpack.from_dlpack(got[1].to_dlpack())
     assert max_abs(host(probs), host(want[1])) < 1e-5
-    # without output_attentions the probabilities stay internal and the result is unchanged
+    # without output_attentions the probabilities stay internal (larger batches take the one-kernel attention then)
     got2 = attn(x, ext)
-    assert len(got2) == 1 and max_abs(host(got2[0]), host(got[0])) == 0
+    assert len(got2) == 1 and max_abs(host(got2[0]), host(got[0])) < 1e-5
 
 
 def test_bert_layer_vs_oracle_and_huggingface(tt, oracle):

@@ -34,13 +34,23 @@ void BertAttention::EnforceShapeAndType() const {
   TT_ENFORCE_EQ(layernorm_beta_.numel(), dense_weight_.shape(0), "LayerNorm bias size mismatch");
 }
 
-bool MultiHeadedAttention::UseFusedCore(const Tensor& attention_mask, const Tensor* att_score, int64_t head_dim, int dtype) {
+bool MultiHeadedAttention::UseFusedCore(const Tensor& attention_mask, const Tensor* att_score, int64_t head_dim, int dtype,
+                                        int64_t batch, int64_t seq, int64_t heads) {
   bool mask_is_key_mask = true;
   if (!attention_mask.is_null()) {
     mask_is_key_mask = attention_mask.n_dim() == 2 || (attention_mask.n_dim() == 3 && attention_mask.shape(1) == 1) ||
                        (attention_mask.n_dim() == 4 && attention_mask.shape(2) == 1);
   }
-  return att_score == nullptr && head_dim == 64 && (dtype == TTMI_F16 || dtype == TTMI_BF16) && mask_is_key_mask;
+  bool dtype_ok = dtype == TTMI_F16 || dtype == TTMI_BF16;
+  if (dtype == TTMI_F32 && batch > 0) {
+    // fp32 has the fused kernel for dense batches (batch = 0: a packed one), with V transposed, and it is bound by the
+    // matrix pipe: a wavefront's 32 queries cost 3.4 us per 64 keys.  It beats the three launches of the chain (18 us)
+    // when the sequence is short or when there are wavefronts for half the SIMDs (1024 on this chip); and a QKV
+    // projection of up to 192 rows is cut along K, which the transposed-V epilogue cannot be.
+    const int64_t wave_blocks = batch * heads * ((seq + 31) / 32);
+    dtype_ok = batch * seq > 192 && (seq <= 128 || wave_blocks >= 512);
+  }
+  return att_score == nullptr && head_dim == 64 && dtype_ok && mask_is_key_mask;
 }
 
 static int64_t RoundUp8(int64_t n) { return (n + 7) / 8 * 8; }
@@ -189,7 +199,7 @@ void MultiHeadedAttention::operator()(const Tensor& key_tensor, const Tensor& va
     MultiHeadedAttention::EnforceShapeAndType();
     // with the fused core V is kept transposed, [B,h,d,pitch]: its tiles are then plain copies.
     // A key/value cache needs the row-major layout (it is appended along the sequence).
-    if (layer_cache.empty() && UseFusedCore(attention_mask, att_score, d, dt)) v_pitch = RoundUp8(seq);
+    if (layer_cache.empty() && UseFusedCore(attention_mask, att_score, d, dt, batch, seq, heads)) v_pitch = RoundUp8(seq);
     q_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/q/Reshape");
     k_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/k/Reshape");
     if (v_pitch > 0) v_.ReshapeAs(query_tensor.dtype(), {batch, heads, d, v_pitch}, dev, dev_id, "self/v/Reshape");

@@ -71,7 +71,9 @@ class MultiHeadedAttention {
                      bool post_add_input, bool is_trans_weight) const;
   // The whole attention core runs as one kernel when nobody asks for the probabilities
   // (fp16/bf16, head size 64, additive key mask broadcast over the query rows).
-  static bool UseFusedCore(const core::Tensor& attention_mask, const core::Tensor* att_score, int64_t head_dim, int dtype);
+  // batch, seq, heads: the shape of a dense batch (fp32 takes the fused kernel only for those, and only where it pays)
+  static bool UseFusedCore(const core::Tensor& attention_mask, const core::Tensor* att_score, int64_t head_dim, int dtype,
+                           int64_t batch = 0, int64_t seq = 0, int64_t heads = 0);
 
   core::Tensor k_weight_, k_bias_, v_weight_, v_bias_, q_weight_, q_bias_;
   core::Tensor dense_weight_, dense_bias_, qkv_weight_, qkv_bias_;

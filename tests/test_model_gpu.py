@@ -94,7 +94,8 @@ def test_bert_layer_vs_oracle_and_huggingface(tt, oracle):
     assert max_abs(host(got[0]), host(hf)) < 1e-3  # bert_layer_test.py:82-86
 
 
-@pytest.mark.parametrize("B,S", [(2, 50), (4, 4), (1, 16)])  # bert_model_test.py:91-92
+# bert_model_test.py:91-92; (6, 40) and (8, 200) are shapes at which fp32 takes the one-kernel attention
+@pytest.mark.parametrize("B,S", [(2, 50), (4, 4), (1, 16), (6, 40), (8, 200)])
 def test_bert_model_fp32_vs_huggingface(tt, B, S):
     model, cfg = _hf_bert(4, seed=B + S)
     tmodel = tt.BertModel.from_torch(model, torch.device("cuda:0"), "turbo")

@@ -53,7 +53,7 @@ constexpr int lds_bytes() {
 }
 
 template <int NW>
-__global__ __launch_bounds__(NW * 64) void fused_attention_f32_kernel(const float* __restrict__ q, const float* __restrict__ k,
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void fused_attention_f32_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                                       const float* __restrict__ v, const float* __restrict__ mask,
                                                                       float* __restrict__ out, int heads, int seq, int v_pitch,
                                                                       float scale_log2e, float inv_scale) {

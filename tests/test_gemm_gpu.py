@@ -576,9 +576,10 @@ def test_fused_attention_vs_unfused_oracle(ttmi, oracle, attention_waves, dt, B,
 @pytest.mark.parametrize("B,h,S,masked", [(2, 3, 128, True), (1, 2, 512, False), (3, 2, 100, True), (2, 1, 37, True),
                                          (1, 1, 500, True), (2, 12, 64, False), (1, 2, 1, False), (1, 1, 700, True),
                                          (3, 2, 260, True), (2, 2, 63, False)])
-def test_fused_attention_fp32_vs_unfused_oracle(ttmi, oracle, attention_waves, B, h, S, masked):
-    """The fp32 form of the one-kernel attention (32x32x2 fp32 matrix instructions, V transposed with NaN in its pad
-    columns) against the oracle's four-step chain, to fp32 accuracy: nothing is rounded to 16 bits on the way."""
+@pytest.mark.parametrize("v_transposed", [False, True])
+def test_fused_attention_fp32_vs_unfused_oracle(ttmi, oracle, attention_waves, B, h, S, masked, v_transposed):
+    """The fp32 form of the one-kernel attention (32x32x2 fp32 matrix instructions; V row-major, or transposed with NaN
+    in its pad columns) against the oracle's four-step chain, to fp32 accuracy: nothing is rounded to 16 bits on the way."""
     rng = np.random.default_rng(S + 3 * B)
     d = 64
     Q, K, V = (rng.standard_normal((B, h, S, d), np.float32) for _ in range(3))
@@ -588,7 +589,7 @@ def test_fused_attention_fp32_vs_unfused_oracle(ttmi, oracle, attention_waves, B
         mask[0, ..., S // 2 + 1:] = -10000.0
         mask[-1, ..., :S // 3] = -10000.0
     dQ, dK = dev(Q, "f32"), dev(K, "f32")
-    dV, pitch = _v_operand(V, "f32", True)
+    dV, pitch = _v_operand(V, "f32", v_transposed)
     out = torch.full((B, S, h * d), 9.0, dtype=torch.float32, device="cuda")
     ok(ttmi.ttmi_fused_attention(ptr(dQ), ptr(dK), ptr(dV), ptr(dev(mask)) if masked else None, ptr(out), None, B, h, S, d,
                                  pitch, 0.125, TTMI_DTYPES["f32"], stream()))
@@ -596,8 +597,9 @@ def test_fused_attention_fp32_vs_unfused_oracle(ttmi, oracle, attention_waves, B
     prob = oracle.apply_mask_and_softmax(score, mask, 1.0, True)
     want = oracle.transpose_for_score(oracle.batch_matmul(prob, V, False)).reshape(B, S, h * d)
     assert max_abs(host(out), want) <= 5e-5
-    # row-major V and packed batches are not built for fp32: refused, not miscomputed
-    assert ttmi.ttmi_fused_attention(ptr(dQ), ptr(dK), ptr(dev(V, "f32")), None, ptr(out), None, B, h, S, d, 0, 0.125,
+    # packed batches are not built for fp32: refused, not miscomputed
+    cu = dev(np.arange(B + 1, dtype=np.int32) * S)
+    assert ttmi.ttmi_fused_attention(ptr(dQ), ptr(dK), ptr(dV), None, ptr(out), ptr(cu), B, h, S, d, pitch, 0.125,
                                      TTMI_DTYPES["f32"], stream()) != 0
 
 

@@ -551,9 +551,10 @@ def test_quantized_bert_layer_vs_oracle_scheme(tt, oracle):
     want = _oracle_qlayer(oracle, host(x), host(ext), w, heads)
     # identical integer arithmetic; fp32 differences upstream (1e-7) can move an activation across a
     # rounding boundary, i.e. one int8 step in one element, hence not bit-exact end to end: almost
-    # all elements agree to fp32 accuracy and the rare flipped step stays small
+    # all elements agree to fp32 accuracy and the rare flipped step stays small (the mean is the flipped steps: 2.1e-5
+    # with the one-kernel fp32 attention, whose sums run in another order than the oracle's chain, 1.9e-5 without)
     diff = np.abs(got - want)
-    assert float(diff.mean()) < 2e-5 and float((diff > 1e-4).mean()) < 0.02 and diff.max() < 5e-2
+    assert float(diff.mean()) < 3e-5 and float((diff > 1e-4).mean()) < 0.02 and diff.max() < 5e-2
     with torch.no_grad():
         fp32 = layer(x, attention_mask=ext)
     fp32 = host(fp32[0] if isinstance(fp32, tuple) else fp32)

@@ -344,7 +344,7 @@ __global__ __launch_bounds__(NW * 64, 16 / NW) void fused_attention_kernel(const
 }  // namespace ttmi
 
 namespace ttmi {
-// attention_f32.hip: the fp32 form (V transposed, dense batch)
+// attention_f32.hip: the fp32 form (dense batch)
 int fused_attention_f32(const float* q, const float* k, const float* v, const float* mask, float* out, int64_t batch,
                         int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, hipStream_t s);
 }  // namespace ttmi
@@ -359,8 +359,7 @@ int ttmi_fused_attention(const void* q, const void* k, const void* v, const floa
   TTMI_REQUIRE(q && k && v && out, "null tensor");
   TTMI_REQUIRE(head_dim == kD, "fused attention is built for head_dim 64");
   TTMI_REQUIRE(dtype == TTMI_F16 || dtype == TTMI_BF16 || dtype == TTMI_F32, "fused attention is built for fp16 / bf16 / fp32");
-  TTMI_REQUIRE(dtype != TTMI_F32 || (v_seq_pitch > 0 && cu_seqlens == nullptr),
-               "fp32 fused attention takes a transposed V (v_seq_pitch > 0) and a dense batch");
+  TTMI_REQUIRE(dtype != TTMI_F32 || cu_seqlens == nullptr, "fp32 fused attention takes dense batches only");
   TTMI_REQUIRE(batch > 0 && heads > 0 && seq > 0 && batch * heads < 65536 && seq < (1 << 24), "bad shape");
   TTMI_REQUIRE(v_seq_pitch == 0 || (v_seq_pitch >= seq && v_seq_pitch % 8 == 0 && v_seq_pitch < (1 << 24)),
                "v_seq_pitch must be 0 or a multiple of 8 that is >= seq");

@@ -16,7 +16,8 @@
 // scale*log2(e) folded into the argument, the additive mask (divided by the scale) seeds the score accumulators, the
 // running maximum is exact.  The matrix pipe bounds the kernel (4*S*64 FLOP per query and head at 157 TFLOP/s).
 //
-// V must be given transposed ([B,h,d,pitch], as the QKV epilogue writes it with v_seq_pitch); batches are dense.
+// V may be given transposed ([B,h,d,pitch], as the QKV epilogue writes it with v_seq_pitch: its tiles are then copied)
+// or row-major ([B,h,S,d]: a thread scatters its four values of a key into four V^T rows); batches are dense.
 #include <cstdlib>
 #include <mutex>
 #include <set>
@@ -52,7 +53,7 @@ constexpr int lds_bytes() {
   return tiles > outb ? tiles : outb;
 }
 
-template <int NW>
+template <int NW, bool VT>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void fused_attention_f32_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                                       const float* __restrict__ v, const float* __restrict__ mask,
                                                                       float* __restrict__ out, int heads, int seq, int v_pitch,
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
 
   const float* qb = q + (int64_t)bh * seq * kD;
   const float* kb = k + (int64_t)bh * seq * kD;
-  const float* vb = v + (int64_t)bh * kD * v_pitch;
+  const float* vb = v + (int64_t)bh * kD * (VT ? v_pitch : seq);
 
   // Q fragments: B operand of the first product, chunk 2kk+lhalf of the lane's query row
   floatx4 qf[8];
@@ -105,8 +106,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     _Pragma("unroll") for (int p = 0; p < kPieces; ++p) {                                                           \
       const int r_ = r0 + p * kRowsPerPass;                                                                         \
       kreg[p] = *reinterpret_cast<const floatx4*>(kb + (int64_t)min(key0_ + r_, kv_len - 1) * kD + ch * 4);         \
-      const int ks_ = min(key0_ + ch * 4, v_pitch - 4);                                                             \
-      vreg[p] = *reinterpret_cast<const floatx4*>(vb + (int64_t)r_ * v_pitch + ks_);                                \
+      if (VT) { /* row r_ of V^T, keys 4ch.. of the tile */                                                         \
+        const int ks_ = min(key0_ + ch * 4, v_pitch - 4);                                                           \
+        vreg[p] = *reinterpret_cast<const floatx4*>(vb + (int64_t)r_ * v_pitch + ks_);                              \
+      } else { /* key r_ of the tile, head dimensions 4ch.. */                                                      \
+        vreg[p] = *reinterpret_cast<const floatx4*>(vb + (int64_t)min(key0_ + r_, kv_len - 1) * kD + ch * 4);       \
+      }                                                                                                             \
     }                                                                                                               \
     if (tid < kBKV) {                                                                                               \
       const int key_ = key0_ + tid;                                                                                 \
@@ -124,10 +129,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
       const int r_ = r0 + p * kRowsPerPass;                                                                         \
       *reinterpret_cast<floatx4*>(kt_ + tile_off(r_, ch)) = kreg[p];                                                \
       floatx4 x_ = vreg[p];                                                                                         \
-      if (nv_ < 4) { /* only in the last tile: keys past the end may hold anything, zero them */                    \
-        _Pragma("unroll") for (int w = 0; w < 4; ++w) if (w >= nv_) x_[w] = 0.f;                                    \
+      if (VT) {                                                                                                     \
+        if (nv_ < 4) { /* only in the last tile: keys past the end may hold anything, zero them */                  \
+          _Pragma("unroll") for (int w = 0; w < 4; ++w) if (w >= nv_) x_[w] = 0.f;                                  \
+        }                                                                                                           \
+        *reinterpret_cast<floatx4*>(vt_ + tile_off(r_, ch)) = x_;                                                   \
+      } else { /* V^T[d = 4ch + w][key r_]: float r_ % 4 of chunk r_ / 4 of row d; keys past the end are zero */    \
+        const bool live_ = (tile_) * kBKV + r_ < kv_len;                                                            \
+        _Pragma("unroll") for (int w = 0; w < 4; ++w)                                                               \
+          *reinterpret_cast<float*>(vt_ + tile_off(ch * 4 + w, r_ >> 2) + (r_ & 3) * 4) = live_ ? x_[w] : 0.f;      \
       }                                                                                                             \
-      *reinterpret_cast<floatx4*>(vt_ + tile_off(r_, ch)) = x_;                                                     \
     }                                                                                                               \
     if (tid < kBKV) reinterpret_cast<float*>(smem + 4 * kTile)[(stage_) * kBKV + tid] = mreg;                       \
   } while (0)
@@ -249,19 +260,24 @@ int fused_attention_f32(const float* q, const float* k, const float* v, const fl
     TTMI_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> lock(mu);
     if (done.count(dev) == 0) {
-      TTMI_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_attention_f32_kernel<8>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<8>()));
-      TTMI_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_attention_f32_kernel<4>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<4>()));
+      const void* kernels[4] = {reinterpret_cast<const void*>(&fused_attention_f32_kernel<8, true>),
+                                reinterpret_cast<const void*>(&fused_attention_f32_kernel<8, false>),
+                                reinterpret_cast<const void*>(&fused_attention_f32_kernel<4, true>),
+                                reinterpret_cast<const void*>(&fused_attention_f32_kernel<4, false>)};
+      for (const void* kern : kernels)
+        TTMI_HIP(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<8>()));
       done.insert(dev);
     }
   }
-  if (nw == 8)
-    hipLaunchKernelGGL((fused_attention_f32_kernel<8>), grid, dim3(512), lds_bytes<8>(), s, q, k, v, mask, out, (int)heads,
-                       (int)seq, (int)v_seq_pitch, sl2, inv_scale);
-  else
-    hipLaunchKernelGGL((fused_attention_f32_kernel<4>), grid, dim3(256), lds_bytes<4>(), s, q, k, v, mask, out, (int)heads,
-                       (int)seq, (int)v_seq_pitch, sl2, inv_scale);
+#define TTMI_FA32_LAUNCH(NW, VT)                                                                                      \
+  hipLaunchKernelGGL((fused_attention_f32_kernel<NW, VT>), grid, dim3(NW * 64), lds_bytes<NW>(), s, q, k, v, mask, out, \
+                     (int)heads, (int)seq, (int)v_seq_pitch, sl2, inv_scale)
+  if (nw == 8) {
+    if (v_seq_pitch > 0) TTMI_FA32_LAUNCH(8, true); else TTMI_FA32_LAUNCH(8, false);
+  } else {
+    if (v_seq_pitch > 0) TTMI_FA32_LAUNCH(4, true); else TTMI_FA32_LAUNCH(4, false);
+  }
+#undef TTMI_FA32_LAUNCH
   return launch_status("fused_attention_f32_kernel");
 }
 

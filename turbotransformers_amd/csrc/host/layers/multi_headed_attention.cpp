@@ -43,12 +43,11 @@ bool MultiHeadedAttention::UseFusedCore(const Tensor& attention_mask, const Tens
   }
   bool dtype_ok = dtype == TTMI_F16 || dtype == TTMI_BF16;
   if (dtype == TTMI_F32 && batch > 0) {
-    // fp32 has the fused kernel for dense batches (batch = 0: a packed one), with V transposed, and it is bound by the
-    // matrix pipe: a wavefront's 32 queries cost 3.4 us per 64 keys.  It beats the three launches of the chain (18 us)
-    // when the sequence is short or when there are wavefronts for half the SIMDs (1024 on this chip); and a QKV
-    // projection of up to 192 rows is cut along K, which the transposed-V epilogue cannot be.
+    // fp32 has the fused kernel for dense batches (batch = 0: a packed one), and it is bound by the matrix pipe: a
+    // wavefront's 32 queries cost 3.4 us per 64 keys.  It beats the three launches of the chain (18 us) when the
+    // sequence is short or when there are wavefronts for half the SIMDs (1024 on this chip).
     const int64_t wave_blocks = batch * heads * ((seq + 31) / 32);
-    dtype_ok = batch * seq > 192 && (seq <= 128 || wave_blocks >= 512);
+    dtype_ok = seq <= 128 || wave_blocks >= 512;
   }
   return att_score == nullptr && head_dim == 64 && dtype_ok && mask_is_key_mask;
 }
@@ -195,11 +194,16 @@ void MultiHeadedAttention::operator()(const Tensor& key_tensor, const Tensor& va
   const Tensor* k_used = &k_;
   const Tensor* v_used = &v_;
   int64_t v_pitch = 0;
+  bool fused_core = false;
   if (is_self) {
     MultiHeadedAttention::EnforceShapeAndType();
     // with the fused core V is kept transposed, [B,h,d,pitch]: its tiles are then plain copies.
     // A key/value cache needs the row-major layout (it is appended along the sequence).
-    if (layer_cache.empty() && UseFusedCore(attention_mask, att_score, d, dt, batch, seq, heads)) v_pitch = RoundUp8(seq);
+    // (fp32 with up to 192 rows keeps V row-major: that QKV projection is cut along K, which the transposed-V
+    // epilogue cannot be, and the fp32 kernel takes either layout)
+    const bool fused_self = layer_cache.empty() && UseFusedCore(attention_mask, att_score, d, dt, batch, seq, heads);
+    if (fused_self && !(dt == TTMI_F32 && batch * seq <= 192)) v_pitch = RoundUp8(seq);
+    fused_core = fused_self;
     q_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/q/Reshape");
     k_.ReshapeAs(query_tensor.dtype(), {batch, heads, seq, d}, dev, dev_id, "self/k/Reshape");
     if (v_pitch > 0) v_.ReshapeAs(query_tensor.dtype(), {batch, heads, d, v_pitch}, dev, dev_id, "self/v/Reshape");
@@ -257,10 +261,10 @@ void MultiHeadedAttention::operator()(const Tensor& key_tensor, const Tensor& va
       }
     }
   }
-  const int64_t key_seq = v_pitch > 0 ? seq : k_used->shape(2);
-  TT_ENFORCE_EQ(v_pitch > 0 ? seq : v_used->shape(2), key_seq, "keys and values differ in length");
+  const int64_t key_seq = fused_core ? seq : k_used->shape(2);
+  TT_ENFORCE_EQ(fused_core ? seq : v_used->shape(2), key_seq, "keys and values differ in length");
 
-  AttentionTail(query_tensor, attention_mask, output, att_score, batch, seq, key_seq, *k_used, *v_used, nullptr, v_pitch > 0, v_pitch,
+  AttentionTail(query_tensor, attention_mask, output, att_score, batch, seq, key_seq, *k_used, *v_used, nullptr, fused_core, v_pitch,
                 post_layernorm, post_add_input, is_trans_weight);
 }
 

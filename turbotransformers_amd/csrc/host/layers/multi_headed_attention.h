@@ -60,6 +60,12 @@ class MultiHeadedAttention {
                   bool pre_layernorm = false, bool post_layernorm = false, bool post_add_input = false,
                   bool is_trans_weight = false) const;
 
+  // The whole attention core runs as one kernel when nobody asks for the probabilities
+  // (head size 64, additive key mask broadcast over the query rows).
+  // batch, seq, heads: the shape of a dense batch (fp32 takes the fused kernel only for those, and only where it pays)
+  static bool UseFusedCore(const core::Tensor& attention_mask, const core::Tensor* att_score, int64_t head_dim, int dtype,
+                           int64_t batch = 0, int64_t seq = 0, int64_t heads = 0);
+
  protected:
   // Everything after q/k/v exist, shared by the dense and the smart-batch layers.
   // `fused_core`: the one-kernel attention core runs; `v_pitch` > 0: v holds V transposed, [B,h,d,v_pitch].
@@ -69,11 +75,6 @@ class MultiHeadedAttention {
                      const core::Tensor& v, const std::vector<int64_t>* seq_list, bool fused_core, int64_t v_pitch,
                      bool post_layernorm,
                      bool post_add_input, bool is_trans_weight) const;
-  // The whole attention core runs as one kernel when nobody asks for the probabilities
-  // (fp16/bf16, head size 64, additive key mask broadcast over the query rows).
-  // batch, seq, heads: the shape of a dense batch (fp32 takes the fused kernel only for those, and only where it pays)
-  static bool UseFusedCore(const core::Tensor& attention_mask, const core::Tensor* att_score, int64_t head_dim, int dtype,
-                           int64_t batch = 0, int64_t seq = 0, int64_t heads = 0);
 
   core::Tensor k_weight_, k_bias_, v_weight_, v_bias_, q_weight_, q_bias_;
   core::Tensor dense_weight_, dense_bias_, qkv_weight_, qkv_bias_;

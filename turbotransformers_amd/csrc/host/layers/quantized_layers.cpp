@@ -4,6 +4,7 @@
 
 #include "core/device_context.h"
 #include "layers/kernels.h"
+#include "layers/multi_headed_attention.h"
 #include "ttmi.h"
 
 namespace turbo_transformers {
@@ -89,13 +90,26 @@ void QuantizedBertAttention::operator()(const Tensor& input_tensor, const Tensor
   k_.Reshape<float>({B, heads_, S, d}, dev, id, "self/k/Reshape");
   v_.Reshape<float>({B, heads_, S, d}, dev, id, "self/v/Reshape");
   qkv_.ProjectToHeads(input_tensor, qkv_bias_, S, heads_, &q_, &k_, &v_);
+  merged_.Reshape<float>({B, S, H}, dev, id, "batch_gemm4/Reshape");
+  if (MultiHeadedAttention::UseFusedCore(attention_mask, attn, d, TTMI_F32, B, S, heads_)) {
+    // nobody asked for the probabilities: the fp32 one-kernel attention (row-major V) in place of the four launches
+    const float* mask = nullptr;
+    if (!attention_mask.is_null()) {
+      TT_ENFORCE_EQ(attention_mask.numel(), B * S, "attention mask has the wrong size");
+      mask = attention_mask.data<float>();
+    }
+    TT_DEVICE_CALL(ttmi_fused_attention(q_.raw(), k_.raw(), v_.raw(), mask, merged_.mutable_raw(), nullptr, B, heads_, S, d, 0,
+                                        1.0f / std::sqrt((float)d), TTMI_F32, Stream()));
+    dense_(merged_, output);
+    kernels::AddBiasLayerNorm<float>(input_tensor, dense_bias_, ln_weight_, ln_bias_, output, 1e-12f);
+    return;
+  }
   Tensor* score = attn != nullptr ? attn : &score_scratch_;
   score->Reshape<float>({B, heads_, S, S}, dev, id, "batch_gemm3/Reshape");
   kernels::BatchMatMul(q_, false, k_, true, 1.0f / std::sqrt((float)d), score, 0.f);
   kernels::ApplyMaskAndSoftmax(score, attention_mask, 1.0f);
   ctx_.Reshape<float>({B, heads_, S, d}, dev, id, "ApplyMaskAndSoftmax/Reshape");
   kernels::BatchMatMul(*score, false, v_, false, 1.0f, &ctx_, 0.f);
-  merged_.Reshape<float>({B, S, H}, dev, id, "batch_gemm4/Reshape");
   kernels::TransposeForScore(&merged_, ctx_);
   dense_(merged_, output);
   kernels::AddBiasLayerNorm<float>(input_tensor, dense_bias_, ln_weight_, ln_bias_, output, 1e-12f);

@@ -279,7 +279,7 @@ TTMI_API int ttmi_gemm_batched_heads(const void* a, const void* b, void* c, int6
                                      int64_t c_head, int64_t batch, int trans_b, float alpha, float beta,
                                      int dtype, void* stream);
 
-/* Self-attention core in one kernel, for head_dim 64 and fp16/bf16/fp32 (fp32: dense batches only, cu_seqlens NULL):
+/* Self-attention core in one kernel, for head_dim 64 and fp16/bf16/fp32:
  *   out[b, s, head*64 + :] = softmax(scale * q[b,head,s,:] k[b,head]^T + mask[b,:]) v[b,head]
  * q,k,v are [B,h,S,64]; `mask` is an additive fp32 [B,S] key mask or NULL; `out` is [B,S,h*64].
  * It replaces BatchMatMul + ApplyMaskAndSoftmax + BatchMatMul + TransposeForScore

@@ -344,9 +344,9 @@ __global__ __launch_bounds__(NW * 64, 16 / NW) void fused_attention_kernel(const
 }  // namespace ttmi
 
 namespace ttmi {
-// attention_f32.hip: the fp32 form (dense batch)
-int fused_attention_f32(const float* q, const float* k, const float* v, const float* mask, float* out, int64_t batch,
-                        int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, hipStream_t s);
+// attention_f32.hip: the fp32 form
+int fused_attention_f32(const float* q, const float* k, const float* v, const float* mask, float* out, const int32_t* cu,
+                        int64_t batch, int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, hipStream_t s);
 }  // namespace ttmi
 
 using namespace ttmi;
@@ -359,7 +359,6 @@ int ttmi_fused_attention(const void* q, const void* k, const void* v, const floa
   TTMI_REQUIRE(q && k && v && out, "null tensor");
   TTMI_REQUIRE(head_dim == kD, "fused attention is built for head_dim 64");
   TTMI_REQUIRE(dtype == TTMI_F16 || dtype == TTMI_BF16 || dtype == TTMI_F32, "fused attention is built for fp16 / bf16 / fp32");
-  TTMI_REQUIRE(dtype != TTMI_F32 || cu_seqlens == nullptr, "fp32 fused attention takes dense batches only");
   TTMI_REQUIRE(batch > 0 && heads > 0 && seq > 0 && batch * heads < 65536 && seq < (1 << 24), "bad shape");
   TTMI_REQUIRE(v_seq_pitch == 0 || (v_seq_pitch >= seq && v_seq_pitch % 8 == 0 && v_seq_pitch < (1 << 24)),
                "v_seq_pitch must be 0 or a multiple of 8 that is >= seq");
@@ -389,8 +388,8 @@ int ttmi_fused_attention(const void* q, const void* k, const void* v, const floa
   const float sl2 = scale * 1.4426950408889634f, inv_scale = 1.0f / scale;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == TTMI_F32)
-    return fused_attention_f32((const float*)q, (const float*)k, (const float*)v, mask, (float*)out, batch, heads, seq,
-                               v_seq_pitch, scale, nw, s);
+    return fused_attention_f32((const float*)q, (const float*)k, (const float*)v, mask, (float*)out, cu_seqlens, batch, heads,
+                               seq, v_seq_pitch, scale, nw, s);
 #define TTMI_FA_LAUNCH(T, PACKED, VT, NW)                                                                              \
   hipLaunchKernelGGL((fused_attention_kernel<T, PACKED, VT, NW>), grid, dim3(NW * 64), 0, s, (const T*)q, (const T*)k, \
                      (const T*)v, mask, (T*)out, cu_seqlens, (int)heads, (int)seq, (int)v_seq_pitch, sl2, inv_scale)

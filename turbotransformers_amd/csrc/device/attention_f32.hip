@@ -17,7 +17,9 @@
 // running maximum is exact.  The matrix pipe bounds the kernel (4*S*64 FLOP per query and head at 157 TFLOP/s).
 //
 // V may be given transposed ([B,h,d,pitch], as the QKV epilogue writes it with v_seq_pitch: its tiles are then copied)
-// or row-major ([B,h,S,d]: a thread scatters its four values of a key into four V^T rows); batches are dense.
+// or row-major ([B,h,S,d]: a thread scatters its four values of a key into four V^T rows).  With cu_seqlens q,k,v are
+// the padded tensors of a packed batch (S = longest sequence): keys and queries past a sequence's length are never
+// read and the output is packed [sum(len), h*64].
 #include <cstdlib>
 #include <mutex>
 #include <set>
@@ -53,11 +55,11 @@ constexpr int lds_bytes() {
   return tiles > outb ? tiles : outb;
 }
 
-template <int NW, bool VT>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void fused_attention_f32_kernel(const float* __restrict__ q, const float* __restrict__ k,
-                                                                      const float* __restrict__ v, const float* __restrict__ mask,
-                                                                      float* __restrict__ out, int heads, int seq, int v_pitch,
-                                                                      float scale_log2e, float inv_scale) {
+template <int NW, bool VT, bool PACKED>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void fused_attention_f32_kernel(
+    const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ mask,
+    float* __restrict__ out, const int32_t* __restrict__ cu, int heads, int seq, int v_pitch, float scale_log2e,
+    float inv_scale) {
   static_assert(NW == 4 || NW == 8, "four or eight wavefronts");
   constexpr int kBQ = NW * 32;               // queries per workgroup
   constexpr int kPieces = 1024 / (NW * 64);  // 16-byte pieces of a K (V^T) tile per thread: 64 rows of 16
@@ -70,7 +72,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   const int lrow = lane & 31, lhalf = lane >> 5;
   const int bh = blockIdx.y, b = bh / heads, head = bh - b * heads;
   const int q0 = blockIdx.x * kBQ + wave * 32;
-  const int kv_len = seq;
+  int kv_len = seq, out_row0 = b * seq;
+  if (PACKED) {
+    kv_len = cu[b + 1] - cu[b];
+    out_row0 = cu[b];
+    if ((int)blockIdx.x * kBQ >= kv_len) return;  // whole workgroup is padding
+  }
+  const int q_len = kv_len;  // self attention: as many queries as keys
 
   const float* qb = q + (int64_t)bh * seq * kD;
   const float* kb = k + (int64_t)bh * seq * kD;
@@ -82,7 +90,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     const int qi = q0 + lrow;
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) {
-      if (qi < seq) qf[kk] = *reinterpret_cast<const floatx4*>(qb + (int64_t)qi * kD + (2 * kk + lhalf) * 4);
+      if (qi < q_len) qf[kk] = *reinterpret_cast<const floatx4*>(qb + (int64_t)qi * kD + (2 * kk + lhalf) * 4);
       else qf[kk] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
   }
@@ -203,7 +211,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   };
 
   const int tiles = (kv_len + kBKV - 1) / kBKV;
-  const bool wave_active = q0 < seq;
+  const bool wave_active = q0 < q_len;
   TTMI_FA32_LOAD(0);
   TTMI_FA32_STORE(0, 0);
   __syncthreads();
@@ -238,9 +246,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   for (int p = 0; p < 8; ++p) {
     const int r = p * 4 + (lane >> 4), cchunk = lane & 15;
     const int qi = q0 + r;
-    if (qi < seq) {
+    if (qi < q_len) {
       const floatx4 x = *reinterpret_cast<const floatx4*>(stage_o + r * (kD + 4) + cchunk * 4);
-      *reinterpret_cast<floatx4*>(out + ((int64_t)b * seq + qi) * hd + head * kD + cchunk * 4) = x;
+      *reinterpret_cast<floatx4*>(out + ((int64_t)out_row0 + qi) * hd + head * kD + cchunk * 4) = x;
     }
   }
 }
@@ -248,36 +256,40 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
 }  // namespace
 
 // Launch; arguments were checked by ttmi_fused_attention.
-int fused_attention_f32(const float* q, const float* k, const float* v, const float* mask, float* out, int64_t batch,
-                        int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, hipStream_t s) {
+int fused_attention_f32(const float* q, const float* k, const float* v, const float* mask, float* out, const int32_t* cu,
+                        int64_t batch, int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, hipStream_t s) {
   const dim3 grid((unsigned)ceil_div(seq, nw * 32), (unsigned)(batch * heads));
   const float sl2 = scale * 1.4426950408889634f, inv_scale = 1.0f / scale;
-  {
-    // more than 64 KB of dynamic LDS: the limit is raised once per kernel and device
+  // more than 64 KB of dynamic LDS: the limit is raised once per kernel and device
+  auto launch = [&](auto kern, int threads, int lds) -> int {
     static std::mutex mu;
-    static std::set<int> done;
+    static std::set<std::pair<const void*, int>> done;
     int dev = 0;
     TTMI_HIP(hipGetDevice(&dev));
-    std::lock_guard<std::mutex> lock(mu);
-    if (done.count(dev) == 0) {
-      const void* kernels[4] = {reinterpret_cast<const void*>(&fused_attention_f32_kernel<8, true>),
-                                reinterpret_cast<const void*>(&fused_attention_f32_kernel<8, false>),
-                                reinterpret_cast<const void*>(&fused_attention_f32_kernel<4, true>),
-                                reinterpret_cast<const void*>(&fused_attention_f32_kernel<4, false>)};
-      for (const void* kern : kernels)
-        TTMI_HIP(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<8>()));
-      done.insert(dev);
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      const void* fn = reinterpret_cast<const void*>(kern);
+      if (done.count({fn, dev}) == 0) {
+        TTMI_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        done.insert({fn, dev});
+      }
     }
-  }
-#define TTMI_FA32_LAUNCH(NW, VT)                                                                                      \
-  hipLaunchKernelGGL((fused_attention_f32_kernel<NW, VT>), grid, dim3(NW * 64), lds_bytes<NW>(), s, q, k, v, mask, out, \
-                     (int)heads, (int)seq, (int)v_seq_pitch, sl2, inv_scale)
+    hipLaunchKernelGGL(kern, grid, dim3(threads), lds, s, q, k, v, mask, out, cu, (int)heads, (int)seq, (int)v_seq_pitch, sl2,
+                       inv_scale);
+    return 0;
+  };
+  const bool vt = v_seq_pitch > 0, packed = cu != nullptr;
+  int rc = 0;
+#define TTMI_FA32_CASE(NW, VT, PACKED) rc = launch(&fused_attention_f32_kernel<NW, VT, PACKED>, NW * 64, lds_bytes<NW>())
   if (nw == 8) {
-    if (v_seq_pitch > 0) TTMI_FA32_LAUNCH(8, true); else TTMI_FA32_LAUNCH(8, false);
+    if (vt) { if (packed) TTMI_FA32_CASE(8, true, true); else TTMI_FA32_CASE(8, true, false); }
+    else { if (packed) TTMI_FA32_CASE(8, false, true); else TTMI_FA32_CASE(8, false, false); }
   } else {
-    if (v_seq_pitch > 0) TTMI_FA32_LAUNCH(4, true); else TTMI_FA32_LAUNCH(4, false);
+    if (vt) { if (packed) TTMI_FA32_CASE(4, true, true); else TTMI_FA32_CASE(4, true, false); }
+    else { if (packed) TTMI_FA32_CASE(4, false, true); else TTMI_FA32_CASE(4, false, false); }
   }
-#undef TTMI_FA32_LAUNCH
+#undef TTMI_FA32_CASE
+  if (rc != 0) return rc;
   return launch_status("fused_attention_f32_kernel");
 }
 

@@ -43,9 +43,9 @@ bool MultiHeadedAttention::UseFusedCore(const Tensor& attention_mask, const Tens
   }
   bool dtype_ok = dtype == TTMI_F16 || dtype == TTMI_BF16;
   if (dtype == TTMI_F32 && batch > 0) {
-    // fp32 has the fused kernel for dense batches (batch = 0: a packed one), and it is bound by the matrix pipe: a
-    // wavefront's 32 queries cost 3.4 us per 64 keys.  It beats the three launches of the chain (18 us) when the
-    // sequence is short or when there are wavefronts for half the SIMDs (1024 on this chip).
+    // the fp32 kernel is bound by the matrix pipe: a wavefront's 32 queries cost 3.4 us per 64 keys.  It beats the
+    // three launches of the chain (18 us) when the sequence is short or when there are wavefronts for half the SIMDs
+    // (1024 on this chip).  (batch, seq: of the padded tensors when the batch is a packed one)
     const int64_t wave_blocks = batch * heads * ((seq + 31) / 32);
     dtype_ok = seq <= 128 || wave_blocks >= 512;
   }
@@ -313,7 +313,7 @@ void MultiHeadedAttentionSmartBatch::operator()(const Tensor& key_tensor, const 
   // V stays row-major here: the transposed store needs the row map and a division per group of eight packed rows,
   // and that costs the QKV GEMM more than the scatter costs the attention kernel (20 requests, 6275 tokens:
   // 2.50 against 2.39 ms per forward).
-  const bool fused_core = UseFusedCore(attention_mask, att_score, d, dt);
+  const bool fused_core = UseFusedCore(attention_mask, att_score, d, dt, batch, max_seq, heads);
   Tensor* qkv[3] = {&q_, &k_, &v_};
   const char* names[3] = {"self/q/Reshape", "self/k/Reshape", "self/v/Reshape"};
   for (int i = 0; i < 3; ++i) {

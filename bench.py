@@ -504,6 +504,9 @@ def main():
         extras["smart_batch"] = run_smart_batch(max(10, args.steps // 2), args.warmup)
         r = run_dense("large_bf16_b64_s512", 10, 2)
         extras["large_bf16_b64_s512"] = {k: r[k] for k in ("ms_per_step", "p50_ms", "seq_per_s", "tflops")}
+        if args.workload != "base_f32_b64_s512":  # the reference's own element type at the headline shape
+            r = run_dense("base_f32_b64_s512", 5, 2)
+            extras["base_f32_b64_s512"] = {k: r[k] for k in ("ms_per_step", "p50_ms", "seq_per_s", "tflops", "frac_of_mfma_peak")}
         extras["albert_f16_b8_s256"] = run_albert(30, args.warmup)
         extras["base_int8_b20_s128"] = run_int8(30, args.warmup)
         line["other_workloads"] = extras

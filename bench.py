@@ -15,6 +15,7 @@ HIP events, and the CPU oracle timed on the host cores of the same box.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
     python bench.py --only-extra smart_batch|albert_f16_b8_s256|base_int8_b20_s128   (one other configuration, for profiling)
     python bench.py --grid f16|bf16|f32   (the reference's fixed-length grid, this library beside PyTorch eager)
+    python bench.py --yardstick           (what the box reaches outside this library: MFMA-only loop, hipBLASLt, copies)
 """
 import argparse
 import ctypes
@@ -377,6 +378,191 @@ def kernel_rooflines(dtype="f16", batch=64, seq=512, hidden=768, heads=12, ffn=3
     return res
 
 
+def run_yardstick(iters=20):
+    """What this box reaches with code that is not this library's: the roofs the encoder kernels can be held against
+    besides the published peaks.  Test-time only; nothing here is on a product path.  Prints a markdown report:
+      (a) a loop of nothing but matrix instructions on register operands (ttmi_yardstick_mfma), both instruction
+          shapes, zeros / N(0,1) / N(0,0.02^2) operands, with the shader clock the chip held (read inside the kernel);
+      (b) ttmi_gemm / ttmi_gemm_fused(bias) against torch.nn.functional.linear (hipBLASLt) on the four encoder
+          products of BERT-base and the two FFN products of BERT-large at 64 x 512 tokens, fp16 and bf16, same
+          operands (activations N(0,1), weights N(0,0.02^2)), loops of `iters` launches;
+      (c) the device copy rate: ttmi_convert fp32 -> fp32 (this library's copy kernel) and torch's copy_, 256 MiB and
+          1 GiB per direction.
+    Methodology as the reference's own GEMM micro-benchmark (benchmark/turbo_transformers/layers/kernels/
+    matmul_benchmark.cpp:60-70: warm-up, a timed loop, 2*m*n*k FLOP per launch)."""
+    import torch
+    from turbotransformers_amd import capi
+    lib = capi.load()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    S = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def timed(fn, n=iters):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e3  # us
+
+    import turbo_transformers
+    info = turbo_transformers.cxx.device_info()
+    cus = int(info.get("compute_units", 256))
+    out = ["# Yardsticks of this box (`python3 bench.py --yardstick`)", "",
+           "Device: %s, %d compute units.  Test-time measurements; nothing here is on a product path." % (info["name"], cus), ""]
+
+    # (a) matrix instructions only
+    out += ["## (a) A loop of nothing but matrix instructions (register operands, eight wavefronts per CU)", "",
+            "| type | instruction | operands | TFLOP/s | of 2.5 PFLOP/s | shader clock held (GHz) | matrix-pipe occupancy |",
+            "|---|---|---|---|---|---|---|"]
+    sink = torch.zeros(1, device="cuda")
+    clocks = torch.zeros(2 * cus, dtype=torch.int64, device="cuda")
+    loop_iters = 150000
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    for dtype, tdt, cdt in (("f16", torch.float16, capi.F16), ("bf16", torch.bfloat16, capi.BF16)):
+        pools = {"zeros": torch.zeros(65536, device="cuda", dtype=tdt),
+                 "N(0,1)": torch.randn(65536, device="cuda", generator=gen).to(tdt),
+                 "N(0,0.02^2)": (torch.randn(65536, device="cuda", generator=gen) * 0.02).to(tdt)}
+        for block in (16, 32):
+            for label, pool in pools.items():
+                fn = lambda: capi.check(lib.ttmi_yardstick_mfma(block, cdt, P(pool), loop_iters, cus, P(sink), P(clocks), S()))
+                fn()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1)
+                ck = clocks.view(cus, 2).double().cpu()
+                if os.environ.get("TTMI_BENCH_DEBUG"):
+                    print("yardstick %s %d %s: %.2f ms, shader cycles mean %.3e min %.3e max %.3e, 100 MHz ticks mean %.3e" % (
+                        dtype, block, label, ms, ck[:, 0].mean(), ck[:, 0].min(), ck[:, 0].max(), ck[:, 1].mean()), file=sys.stderr)
+                ghz = float((ck[:, 0] / ck[:, 1]).mean()) * 0.1  # shader cycles per tick of the 100 MHz clock
+                flop = cus * 8 * loop_iters * 262144.0
+                # share of the matrix pipes' cycles at the clock held: a SIMD retires 1024 FLOP per cycle in these types.
+                # (The two counters are read by the first wavefront of each workgroup, which a SIMD serves ahead of its
+                # younger neighbour: their ratio is the clock, but the time is taken from the events around the launch.)
+                occupancy = flop / (ms * 1e-3) / (cus * 4 * 1024.0 * ghz * 1e9)
+                out.append("| %s | %s | %s | %.0f | %.2f | %.2f | %.0f %% |" % (
+                    dtype, "16x16x32" if block == 16 else "32x32x16", label, flop / ms / 1e9, flop / ms / 1e9 / 2500.0, ghz,
+                    100 * occupancy))
+    out.append("")
+
+    # (b) this library's GEMM beside hipBLASLt
+    out += ["## (b) `ttmi_gemm` beside `torch.nn.functional.linear` (hipBLASLt), 32768 rows, loops of %d launches" % iters, "",
+            "Activations N(0,1), weights N(0,0.02^2), the same tensors for both; us per launch (TFLOP/s, share of 2.5 PFLOP/s).", "",
+            "| product | N x K | type | form | this library | hipBLASLt | this / hipBLASLt time |", "|---|---|---|---|---|---|---|"]
+    M = 64 * 512
+    shapes = [("base QKV", 2304, 768), ("base out-proj", 768, 768), ("base FFN1", 3072, 768), ("base FFN2", 768, 3072),
+              ("large FFN1", 4096, 1024), ("large FFN2", 1024, 4096)]
+    for name, N, K in shapes:
+        for dtype, tdt, cdt in (("f16", torch.float16, capi.F16), ("bf16", torch.bfloat16, capi.BF16)):
+            A = torch.randn(M, K, device="cuda", generator=gen).to(tdt)
+            W = (torch.randn(N, K, device="cuda", generator=gen) * 0.02).to(tdt)
+            bias = (torch.randn(N, device="cuda", generator=gen) * 0.02).to(tdt)
+            C = torch.empty(M, N, device="cuda", dtype=tdt)
+            args = capi.EpilogueArgs()
+            args.bias = bias.data_ptr()
+            forms = {"bare": (lambda: capi.check(lib.ttmi_gemm(P(A), P(W), P(C), M, N, K, K, K, N, 1, 1.0, 0.0, cdt, S())),
+                              lambda: torch.nn.functional.linear(A, W)),
+                     "+ bias": (lambda: capi.check(lib.ttmi_gemm_fused(P(A), P(W), P(C), M, N, K, K, K, N, capi.EPI_BIAS,
+                                                                       ctypes.byref(args), cdt, S())),
+                                lambda: torch.nn.functional.linear(A, W, bias))}
+            flop = 2.0 * M * N * K
+            for form, (mine, theirs) in forms.items():
+                us_m, us_t = timed(mine), timed(theirs)
+                out.append("| %s | %d x %d | %s | %s | %.1f (%.0f, %.2f) | %.1f (%.0f, %.2f) | %.2f |" % (
+                    name, N, K, dtype, form, us_m, flop / us_m / 1e6, flop / us_m / 1e6 / 2500.0, us_t, flop / us_t / 1e6,
+                    flop / us_t / 1e6 / 2500.0, us_m / us_t))
+            del A, W, C
+    out.append("")
+
+    # (c) copies
+    out += ["## (c) Device copy rate (bytes read + bytes written, over the time of a launch)", "",
+            "| copy | bytes each way | us | GB/s | of 8 TB/s |", "|---|---|---|---|---|"]
+    for mib in (256, 1024):
+        n = mib << 18  # fp32 elements
+        src = torch.randn(n, device="cuda")
+        dst = torch.empty_like(src)
+        for label, fn in (("ttmi_convert fp32 -> fp32", lambda: capi.check(lib.ttmi_convert(P(src), capi.F32, P(dst), capi.F32, n, S()))),
+                          ("torch copy_", lambda: dst.copy_(src))):
+            us = timed(fn)
+            gbs = 2.0 * n * 4 / us / 1e3
+            out.append("| %s | %d MiB | %.1f | %.0f | %.2f |" % (label, mib, us, gbs, gbs / PEAK_HBM_GBS))
+        del src, dst
+    print("\n".join(out))
+
+
+def run_ffn2_probe(iters=20, batch=64, seq=512, hidden=768, ffn=3072):
+    """Why the second FFN product (32768 x 768 x 3072, fp16) takes longer inside the forward than in a loop of itself:
+    loops of short kernel sequences through the C ABI, timed with events around the whole loop (us per pass).  The
+    interaction cost of a pair is t(pair) - t(first alone) - t(second alone).  `own` = FFN2 reads what the FFN1 launch
+    in front of it has just written (201 MB); `other` = it reads a second buffer of the same statistics that nothing
+    writes, so that only clocks and caches, not the data dependency, tie the two launches together."""
+    import torch
+    from turbotransformers_amd import capi
+    lib = capi.load()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    S = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    T, H, F = batch * seq, hidden, ffn
+    tdt, cdt = torch.float16, capi.F16
+    x = torch.randn(T, H, device="cuda").to(tdt)
+    w1, w2 = (torch.randn(F, H, device="cuda") * 0.02).to(tdt), (torch.randn(H, F, device="cuda") * 0.02).to(tdt)
+    b1, bh, gam = torch.zeros(F, device="cuda", dtype=tdt), torch.zeros(H, device="cuda", dtype=tdt), torch.ones(H, device="cuda", dtype=tdt)
+    own = torch.empty(T, F, device="cuda", dtype=tdt)
+    out, res = torch.empty(T, H, device="cuda", dtype=tdt), torch.randn(T, H, device="cuda").to(tdt)
+    args = capi.EpilogueArgs()
+    args.bias, args.act = b1.data_ptr(), capi.ACT_GELU
+    ffn1 = lambda: capi.check(lib.ttmi_gemm_fused(P(x), P(w1), P(own), T, F, H, H, H, F, capi.EPI_BIAS_ACT, ctypes.byref(args), cdt, S()))
+    ffn1()
+    other = own.clone()
+    ffn2 = lambda a: (lambda: capi.check(lib.ttmi_gemm(P(a), P(w2), P(out), T, H, F, F, F, H, 1, 1.0, 0.0, cdt, S())))
+    ln = lambda: capi.check(lib.ttmi_add_bias_layer_norm(P(out), P(res), P(bh), P(gam), P(bh), T, H, 1e-12, cdt, S()))
+    copy_src, copy_dst = torch.randn(64 << 20, device="cuda"), torch.empty(64 << 20, device="cuda")
+    flush = lambda: capi.check(lib.ttmi_convert(P(copy_src), capi.F32, P(copy_dst), capi.F32, 64 << 20, S()))  # 512 MB through the caches
+
+    def timed(fns):
+        for _ in range(3):
+            for fn in fns:
+                fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            for fn in fns:
+                fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters * 1e3
+
+    cases = [("FFN2 (other)", [ffn2(other)]), ("FFN1", [ffn1]), ("LayerNorm", [ln]), ("copy 2 x 256 MiB", [flush]),
+             ("FFN1, FFN2 (own)", [ffn1, ffn2(own)]), ("FFN1, FFN2 (other)", [ffn1, ffn2(other)]),
+             ("LayerNorm, FFN2 (other)", [ln, ffn2(other)]), ("copy, FFN2 (other)", [flush, ffn2(other)]),
+             ("LayerNorm, FFN1, FFN2 (own), LayerNorm", [ln, ffn1, ffn2(own), ln]),
+             ("FFN2 (other), FFN2 (other)", [ffn2(other), ffn2(other)])]
+    t = {}
+    out_lines = ["# The second FFN product inside the forward and alone (`python3 bench.py --ffn2-probe`)", "",
+                 "fp16, %d x %d tokens; loops of %d passes of each sequence, us per pass (events around the whole loop)." % (batch, seq, iters), "",
+                 "| sequence | us per pass | sum of its parts alone | interaction |", "|---|---|---|---|"]
+    for rnd in range(2):  # two rounds, the second is reported: clocks and caches settled
+        for name, fns in cases:
+            t[name] = timed(fns)
+    single = {"FFN2 (own)": t["FFN2 (other)"], "FFN2 (other)": t["FFN2 (other)"], "FFN1": t["FFN1"], "LayerNorm": t["LayerNorm"],
+              "copy": t["copy 2 x 256 MiB"]}
+    for name, _ in cases:
+        parts = [p.strip() for p in name.split(",")]
+        if len(parts) == 1:
+            out_lines.append("| %s | %.1f | | |" % (name, t[name]))
+        else:
+            alone = sum(single[p] for p in parts)
+            out_lines.append("| %s | %.1f | %.1f | %+.1f |" % (name, t[name], alone, t[name] - alone))
+    print("\n".join(out_lines))
+
+
 def cpu_baseline(seqs=4, seq=512, repeats=2):
     """The CPU oracle (an in-repo restatement of the reference's CPU branch: OpenMP loops + cblas_sgemm)
     on a bounded sample of the headline workload: `seqs` of the 64 sequences, all 12 layers, fp32; timed with 4 and
@@ -435,6 +621,12 @@ def main():
                     help="profiling helper: run just this other configuration of the metric, print its figures, exit")
     ap.add_argument("--grid", default=None, choices=["f16", "bf16", "f32"],
                     help="time the reference's fixed-length grid (batch 1/20 x 10..500 tokens) beside PyTorch eager, print it as JSON and exit")
+    ap.add_argument("--yardstick", action="store_true",
+                    help="print what this box reaches outside this library (a loop of matrix instructions, hipBLASLt on "
+                         "the encoder's products, copy rates) as a markdown report and exit")
+    ap.add_argument("--ffn2-probe", action="store_true",
+                    help="time the second FFN product alone and behind the kernels that precede it in the forward "
+                         "(markdown report), exit")
     ap.add_argument("--pmc-kernel", default=None,
                     help="counter-collection helper: run one calibration copy and a few launches of the named kernel "
                          "of the roofline pass (e.g. ffn1_gemm+bias+gelu), print nothing, exit")
@@ -454,6 +646,12 @@ def main():
         return
     if args.grid:
         print(json.dumps(run_grid(args.grid, args.steps, args.warmup)))
+        return
+    if args.yardstick:
+        run_yardstick()
+        return
+    if args.ffn2_probe:
+        run_ffn2_probe()
         return
     if args.only_extra:
         run = {"smart_batch": lambda: run_smart_batch(max(10, args.steps // 2), args.warmup),

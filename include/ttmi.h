@@ -55,6 +55,18 @@ enum ttmi_epilogue {
 
 TTMI_API const char* ttmi_last_error(void);
 
+/* Kernel-selection switches, for A/B timing and for tests that push small or ragged problems through a kernel the
+ * launchers would not pick for them.  No counterpart in the reference (cuBLAS and the CUDA kernels have no such
+ * knob).  Names and values:
+ *   "TTMI_LARGE_TILE"       1 = every eligible 16-bit product on the one-wavefront-per-SIMD GEMM kernel, 0 = none;
+ *   "TTMI_WAVE_KERNEL"      0 = products of at most 128 rows stay on the LDS-tiled kernels;
+ *   "TTMI_ATTENTION_WAVES"  4 / 8 = wavefronts per workgroup of the one-kernel attention;
+ *   "TTMI_STATIC_SCRATCH_LIMIT"  bytes of its buffer ttmi_gemm_bias_layer_norm_static admits (to test its refusal);
+ *   -1 = the launcher decides (the default).
+ * Each switch starts from the environment variable of the same name, which is read once, at the first launch or
+ * the first call of this function; later changes of the environment are not seen. */
+TTMI_API int ttmi_set_kernel_switch(const char* name, int value);
+
 /* Device bring-up and properties.  Replaces core::CUDADeviceContext
  * (turbo_transformers/core/cuda_device_context.cpp:23-46). */
 TTMI_API int ttmi_device_count(int* count);
@@ -135,9 +147,10 @@ TTMI_API int ttmi_gemm_bias_layer_norm(const void* a, const void* w, void* out, 
  * live in a buffer of TTMI_STATIC_SCRATCH_BYTES that is part of the library's device image (every GPU the
  * library runs on holds it until the process ends) instead of the per-stream workspace ttmi_gemm_bias_layer_norm
  * allocates on first use.  The call reaches no hipMalloc / hipFree.  A problem whose K slices need more than
- * that buffer (slices * m * n * 4 bytes; m = 2560, n = 768, k = 3072 in four slices is the largest the encoder
- * configurations produce) is refused with TTMI_EINVAL; problems large enough to run unsplit need no scratch
- * and are accepted at any size.  Nothing has to be cleared between calls (every partial tile that is read
+ * that buffer (slices * m * n * 4 bytes; the largest the encoder configurations produce is m = 2560, n = 768,
+ * k = 3072 in three slices, 23.6 MB) is refused with TTMI_EINVAL; problems large enough to run unsplit need no
+ * scratch and are accepted at any size.  The first call on a device resolves the buffer's address and sets kernel
+ * attributes, so make one call outside a graph capture before capturing calls.  Nothing has to be cleared between calls (every partial tile that is read
  * has been written by the same call), but all calls on one GPU share the buffer: calls that overlap in time
  * on one GPU (different streams or threads) race. */
 #define TTMI_STATIC_SCRATCH_BYTES (32u << 20)
@@ -333,6 +346,19 @@ TTMI_API int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, i
 TTMI_API int ttmi_gemm_describe(int64_t m, int64_t n, int64_t k, int epilogue, const ttmi_epilogue_args* args, int dtype,
                                 char* out, size_t capacity);
 
+
+/* Measurement aid, never on a product path: a loop of nothing but matrix instructions on register operands, one
+ * workgroup of eight wavefronts per entry of the grid, to find what the matrix pipes sustain on this chip for a
+ * given kind of operand values.  It plays the part of the reference's GEMM micro-benchmark
+ * (benchmark/turbo_transformers/layers/kernels/matmul_benchmark.cpp:60-70) one level further down.
+ *   block      16 = v_mfma_f32_16x16x32, 32 = v_mfma_f32_32x32x16 (of `dtype` TTMI_F16 or TTMI_BF16);
+ *   operands   device buffer of 65536 elements of `dtype` the operand registers are filled from;
+ *   iters      loop iterations; each is 262144 FLOP per wavefront (eight wavefronts per workgroup);
+ *   sink       one device float (keeps the result alive; not written in practice);
+ *   clocks     device uint64[2 * workgroups]: per workgroup, shader-clock cycles and ticks of the constant
+ *              100 MHz clock spent in the loop (their ratio is the shader clock the chip held). */
+TTMI_API int ttmi_yardstick_mfma(int block, int dtype, const void* operands, int iters, int workgroups, float* sink,
+                                 uint64_t* clocks, void* stream);
 
 /* int8 path (quantized BERT: int8 x int8 -> int32 accumulators, exact).
  * ttmi_quantize_rows_i8: per-tensor symmetric dynamic scale from max|x| over the whole

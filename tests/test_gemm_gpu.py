@@ -89,16 +89,12 @@ def test_fused_epilogues_small_m_long_k(ttmi, oracle, dt):
 
 
 @pytest.fixture
-def large_tile_forced():
-    """TTMI_LARGE_TILE=1 sends every eligible problem to the one-wavefront-per-SIMD kernel whatever its size."""
-    import os
-    old = os.environ.get("TTMI_LARGE_TILE")
-    os.environ["TTMI_LARGE_TILE"] = "1"
+def large_tile_forced(ttmi):
+    """Switch TTMI_LARGE_TILE = 1 sends every eligible problem to the one-wavefront-per-SIMD kernel whatever its
+    size (set through the C ABI: the library reads its environment variables only once)."""
+    ok(ttmi.ttmi_set_kernel_switch(b"TTMI_LARGE_TILE", 1))
     yield
-    if old is None:
-        del os.environ["TTMI_LARGE_TILE"]
-    else:
-        os.environ["TTMI_LARGE_TILE"] = old
+    ok(ttmi.ttmi_set_kernel_switch(b"TTMI_LARGE_TILE", -1))
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
@@ -110,7 +106,6 @@ def test_large_tile_kernel_against_oracle_and_small_tiles(ttmi, oracle, large_ti
     plain and the bias form may differ by the last bit of the output type and no more (the 16x16x32 matrix instruction
     sums the 32 products of a step in another order than the 32x32x16 one: fp32 rounding of the accumulator)."""
     import ctypes
-    import os
     rng = np.random.default_rng(M + N + K)
     A, W = _ab(rng, M, N, K, 1)
     bias = rng.standard_normal(N).astype(np.float32)
@@ -135,12 +130,43 @@ def test_large_tile_kernel_against_oracle_and_small_tiles(ttmi, oracle, large_ti
     assert max_abs(host(got["bias"]), base + rounded(bias, dt)) <= GEMM_TOL[dt] * 3
     assert max_abs(host(got["gelu"]), oracle.add_bias_act(base, rounded(bias, dt), 0)) <= GEMM_TOL[dt] * 3
     if (M, N, K) != (64, 2304, 768):  # that one is cut along K by the other path: another summation order
-        os.environ["TTMI_LARGE_TILE"] = "0"
+        ok(ttmi.ttmi_set_kernel_switch(b"TTMI_LARGE_TILE", 0))
         ulp = 2.0 ** -10 if dt == "f16" else 2.0 ** -7  # one step of the output type, relative to the larger neighbour
         for form in (None, "bias"):
             a, b = host(run(form)), host(got[form])
             assert np.all(np.abs(a - b) <= ulp * np.maximum(np.abs(a), np.abs(b)) + 1e-6)
             assert np.mean(a != b) < 0.05  # and the two mostly agree exactly
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("M", [1, 300, 777, 4100])
+def test_large_tile_kernel_leaves_rows_past_m_alone(ttmi, oracle, large_tile_forced, dt, M):
+    """The last tile row of the 256-row tiles is ragged for every one of these M.  C lives inside a larger tensor
+    with 256 sentinel rows behind row M (and 8 in front of row 0): the kernel's row-major stores, plain, bias and
+    bias + GELU, must leave every sentinel as it was, and rows 0..M-1 must still be the product."""
+    import ctypes
+    N, K, GUARD = 776, 256, 256
+    rng = np.random.default_rng(M)
+    A, W = _ab(rng, M, N, K, 1)
+    bias = rng.standard_normal(N).astype(np.float32)
+    dA, dW, db = dev(A, dt), dev(W, dt), dev(bias, dt)
+    base = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    want = {"plain": base, "bias": base + rounded(bias, dt), "gelu": oracle.add_bias_act(base, rounded(bias, dt), 0)}
+    SENTINEL = -7.0
+    for form in ("plain", "bias", "gelu"):
+        whole = torch.full((8 + M + GUARD, N), SENTINEL, dtype=dA.dtype, device="cuda")
+        C = whole[8:8 + M]
+        if form == "plain":
+            ok(ttmi.ttmi_gemm(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, 1, 1.0, 0.0, TTMI_DTYPES[dt], stream()))
+        else:
+            epi = _epi(bias=db) if form == "bias" else _epi(bias=db, act=capi.ACT_GELU)
+            ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N,
+                                    capi.EPI_BIAS if form == "bias" else capi.EPI_BIAS_ACT, ctypes.byref(epi),
+                                    TTMI_DTYPES[dt], stream()))
+        torch.cuda.synchronize()
+        assert torch.all(whole[:8] == SENTINEL), form
+        assert torch.all(whole[8 + M:] == SENTINEL), "%s: rows past M were written" % form
+        assert max_abs(host(C), want[form]) <= GEMM_TOL[dt] * 3
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
@@ -538,12 +564,13 @@ def _v_operand(V, dt, v_transposed, poison=True):
 
 
 @pytest.fixture(params=["auto", "8"])
-def attention_waves(request, monkeypatch):
+def attention_waves(request, ttmi):
     """Wavefronts per workgroup of the fused attention kernel: its own choice (eight only for long sequences with a workgroup
-    per compute unit, which none of these small shapes has), and eight forced through TTMI_ATTENTION_WAVES."""
+    per compute unit, which none of these small shapes has), and eight forced through the switch TTMI_ATTENTION_WAVES."""
     if request.param != "auto":
-        monkeypatch.setenv("TTMI_ATTENTION_WAVES", request.param)
-    return request.param
+        ok(ttmi.ttmi_set_kernel_switch(b"TTMI_ATTENTION_WAVES", int(request.param)))
+    yield request.param
+    ok(ttmi.ttmi_set_kernel_switch(b"TTMI_ATTENTION_WAVES", -1))
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])

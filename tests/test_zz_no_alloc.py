@@ -43,7 +43,8 @@ def _both(ttmi, dt, M, N, K, seed, fp32_residual=False):
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
 def test_static_scratch_matches_allocating_entry_point_twice_in_a_row(ttmi, dt):
     """Two calls in a row on the same scratch, the second smaller: a split-K shape on the DMA tiles
-    (M = 2560: four slices, 31.5 MB of partial tiles), then one short sequence (M = 128, sixteen slices)."""
+    (M = 2560: three slices, 23.6 MB of partial tiles), then one short sequence (M = 128, a few slices of the
+    one-wavefront-per-tile kernel)."""
     _both(ttmi, dt, 2560, 768, 3072, seed=1)
     _both(ttmi, dt, 128, 768, 3072, seed=2)
     _both(ttmi, dt, 100, 768, 768, seed=3)
@@ -58,3 +59,60 @@ def test_static_scratch_fp32_residual_stream(ttmi, dt):
 def test_static_scratch_unsplit_problems_need_no_scratch(ttmi):
     """A problem large enough to run unsplit uses no partial tiles and is accepted at any size."""
     _both(ttmi, "f16", 8192, 768, 768, seed=6)
+
+
+def test_static_scratch_refuses_what_does_not_fit(ttmi):
+    """With the admitted size lowered to 1 MiB the K slices of 2560 x 768 x 3072 (23.6 MB of partial tiles) no longer
+    fit: the call is refused with TTMI_EINVAL and a message that names both sizes, nothing is launched and `out`
+    keeps its contents; the allocating entry point and a later call with the limit lifted are unaffected."""
+    M, N, K = 2560, 768, 3072
+    rng = np.random.default_rng(7)
+    dA, dW = dev(rng.standard_normal((M, K)).astype(np.float32), "f16"), dev((rng.standard_normal((N, K)) / 55).astype(np.float32), "f16")
+    dres = dev(rng.standard_normal((M, N)).astype(np.float32), "f16")
+    vec = dev(np.ones(N, np.float32), "f16")
+    out = torch.full((M, N), -7.0, dtype=torch.float16, device="cuda")
+    ok(ttmi.ttmi_set_kernel_switch(b"TTMI_STATIC_SCRATCH_LIMIT", 1 << 20))
+    try:
+        rc = ttmi.ttmi_gemm_bias_layer_norm_static(ptr(dA), ptr(dW), ptr(out), ptr(dres), None, ptr(vec), ptr(vec), ptr(vec), None,
+                                                   M, N, K, 1e-12, TTMI_DTYPES["f16"], stream())
+        assert rc == -1  # TTMI_EINVAL
+        msg = ttmi.ttmi_last_error().decode()
+        assert "static scratch buffer" in msg and str(1 << 20) in msg
+        torch.cuda.synchronize()
+        assert torch.all(out == -7.0)
+    finally:
+        ok(ttmi.ttmi_set_kernel_switch(b"TTMI_STATIC_SCRATCH_LIMIT", -1))
+    _both(ttmi, "f16", M, N, K, seed=8)
+
+
+def test_static_scratch_call_under_graph_capture(ttmi):
+    """What the entry point is for: a call recorded into a HIP graph (after one eager call, which resolves the
+    buffer's address and sets the kernel attributes).  The graph is replayed three times with eager work and
+    synchronisations in between and with fresh operands each time; every replay must reproduce the eager result
+    of the allocating entry point bit for bit."""
+    M, N, K = 128, 768, 3072
+    rng = np.random.default_rng(9)
+    new = lambda *shape: dev(rng.standard_normal(shape).astype(np.float32), "f16")
+    dA, dW, dres = new(M, K), dev((rng.standard_normal((N, K)) / 55).astype(np.float32), "f16"), new(M, N)
+    bias, gamma, beta = new(N), new(N), new(N)
+    out, want = (torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda") for _ in range(2))
+
+    def call(fn, dst, s):
+        ok(fn(ptr(dA), ptr(dW), ptr(dst), ptr(dres), None, ptr(bias), ptr(gamma), ptr(beta), None, M, N, K, 1e-12,
+              TTMI_DTYPES["f16"], s))
+
+    call(ttmi.ttmi_gemm_bias_layer_norm_static, out, stream())  # eager first call
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(ttmi.ttmi_gemm_bias_layer_norm_static, out, stream())  # torch's capture stream is current here
+    for turn in range(3):
+        dA.copy_(new(M, K))
+        dres.copy_(new(M, N))
+        out.fill_(float("nan"))
+        call(ttmi.ttmi_gemm_bias_layer_norm, want, stream())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert not torch.isnan(want).any()
+        assert torch.equal(out, want), "replay %d" % turn

@@ -380,10 +380,8 @@ int ttmi_fused_attention(const void* q, const void* k, const void* v, const floa
   const bool fits_four = seq <= 128 || 8 * ceil_div(seq, 256) >= 5 * ceil_div(seq, 128);
   int nw = (fits_four || ceil_div(seq, 128) * batch * heads < (int64_t)cus) ? 4 : 8;
   // TTMI_ATTENTION_WAVES=4 / 8 overrides the choice (A/B timing, and tests of the eight-wavefront form on small shapes)
-  if (const char* force = std::getenv("TTMI_ATTENTION_WAVES")) {
-    if (force[0] == '4') nw = 4;
-    if (force[0] == '8') nw = 8;
-  }
+  const int force = kernel_switch(kSwitchAttentionWaves);
+  if (force == 4 || force == 8) nw = force;
   const dim3 grid((unsigned)ceil_div(seq, nw * 32), (unsigned)(batch * heads));
   const float sl2 = scale * 1.4426950408889634f, inv_scale = 1.0f / scale;
   hipStream_t s = (hipStream_t)stream;

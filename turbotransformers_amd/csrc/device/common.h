@@ -37,6 +37,14 @@ inline int launch_status(const char* what) { return check_hip(hipGetLastError(),
 
 int* async_error_flag();  // device-visible pinned int, 0 = ok
 
+// ---- kernel-selection switches ----------------------------------------------------------
+// Overrides of the launchers' own choices, for A/B timing and for tests of small and ragged shapes.  Each starts
+// from an environment variable read ONCE (first use; a launch never scans the environment) and can be changed
+// afterwards through ttmi_set_kernel_switch.  kSwitchUnset = the launcher decides.
+constexpr int kSwitchUnset = -1;
+enum KernelSwitch { kSwitchLargeTile = 0, kSwitchWaveKernel = 1, kSwitchAttentionWaves = 2, kSwitchStaticScratchLimit = 3, kNumKernelSwitches = 4 };
+int kernel_switch(KernelSwitch which);
+
 // ---- scalar conversion ----------------------------------------------------------------
 template <typename T>
 __device__ __forceinline__ float to_float(T v) { return static_cast<float>(v); }

@@ -236,11 +236,15 @@ int ttmi_gemm_bias_layer_norm_static(const void* a, const void* w, void* out, co
     const int rc = static_scratch(&ws);
     if (rc != 0) return rc;
   }
-  // Every split-K launch below this call takes its partial tiles from the static buffer, or is refused.
+  // Every split-K launch below this call takes its partial tiles from the static buffer, or is refused.  (The
+  // switch lowers the size that is admitted, so that tests reach the refusal with problems of ordinary size.)
+  size_t capacity = kStaticScratchBytes;
+  const int limit = kernel_switch(kSwitchStaticScratchLimit);
+  if (limit >= 0) capacity = std::min(capacity, (size_t)limit);
   struct Install {
-    explicit Install(float* p) { tl_fixed_workspace = FixedWorkspace{p, kStaticScratchBytes}; }
+    Install(float* p, size_t bytes) { tl_fixed_workspace = FixedWorkspace{p, bytes}; }
     ~Install() { tl_fixed_workspace = FixedWorkspace{}; }
-  } install(ws);
+  } install(ws, capacity);
   return gemm_bias_layer_norm_impl(a, w, out, residual, residual_f32, bias, gamma, beta, out_f32, m, n, k, eps, dtype, stream);
 }
 

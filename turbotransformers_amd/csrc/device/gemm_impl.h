@@ -1337,8 +1337,7 @@ constexpr int kWaveDepth = 4;  // K steps a wavefront keeps in flight: 32 loads 
 template <typename T>
 static bool wave_kernel_ok(const GemmArgs& g, int batch, bool aligned) {
   if (sizeof(T) != 2 || !aligned || batch != 1 || g.m > 128 || g.k % (kRowBytes / (int)sizeof(T)) != 0) return false;
-  if (const char* sw = getenv("TTMI_WAVE_KERNEL")) return sw[0] != '0';
-  return true;
+  return kernel_switch(kSwitchWaveKernel) != 0;
 }
 // K slices for it: up to two wavefronts per CU, at least four K steps per slice.
 static int wave_splits(int64_t m, int64_t n, int64_t ksteps) {
@@ -1365,17 +1364,18 @@ static int launch_wave(GemmArgs g, const Epi& epi, hipStream_t s) {
 // `reduce(ws, slices, vec, stream)` launches the kernel that sums the slices and applies the epilogue.
 template <typename T, typename Reduce>
 static int launch_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStream_t s, const Reduce& reduce) {
+  constexpr int kTile = 64, kWaveTile = 32;  // tile edge of the LDS-tiled and of the one-wavefront form
   const bool wave = wave_kernel_ok<T>(g, 1, true);  // callers come here with aligned operands and one problem
   if (wave) splits = std::max(2, wave_splits(g.m, g.n, ksteps));
-  if (describe_only(wave ? "wave" : "reg", wave ? 1 : 4, wave ? 32 : 64, wave ? 32 : 64, splits)) return 0;
-  const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
+  g.k_chunk = (int)ceil_div(ksteps, splits) * bk;
+  const int used = (int)ceil_div(g.k, g.k_chunk);  // slices that actually hold part of K: what is launched
+  if (describe_only(wave ? "wave" : "reg", wave ? 1 : 4, wave ? kWaveTile : kTile, wave ? kWaveTile : kTile, used)) return 0;
+  const size_t bytes = (size_t)used * g.m * g.n * sizeof(float);
   float* ws = nullptr;
   {
     const int rc = splitk_workspace(bytes, s, &ws);
     if (rc != 0) return rc;
   }
-  g.k_chunk = (int)ceil_div(ksteps, splits) * bk;
-  const int used = (int)ceil_div(g.k, g.k_chunk);  // slices that actually hold part of K
   const bool vec = g.n % 4 == 0;
   EpiPartial part{ws, (int64_t)g.m * g.n, g.n, vec};
   if constexpr (sizeof(T) == 2) {
@@ -1387,12 +1387,12 @@ static int launch_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStre
       return launch_status("gemm_wave_splitk");
     }
   }
-  g.tiles_m = (g.m + 63) / 64;
-  g.tiles_n = (g.n + 63) / 64;
+  g.tiles_m = (g.m + kTile - 1) / kTile;
+  g.tiles_n = (g.n + kTile - 1) / kTile;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-  constexpr int LDS = 2 * (64 + 64) * kRowBytes;
+  constexpr int LDS = 2 * (kTile + kTile) * kRowBytes;
   const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
-  hipLaunchKernelGGL((gemm_kernel<T, 64, 64, 2, 2, false, true, 2, EpiPartial>), dim3(grid_x, (unsigned)used, 1), dim3(256), LDS, s,
+  hipLaunchKernelGGL((gemm_kernel<T, kTile, kTile, 2, 2, false, true, 2, EpiPartial>), dim3(grid_x, (unsigned)used, 1), dim3(256), LDS, s,
                      g, part);
   reduce(ws, used, vec, s);
   return launch_status("gemm_splitk");
@@ -1402,22 +1402,23 @@ static int launch_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStre
 // (M = 2560, N = 768, K = 3072: 120 tiles, 48 K steps each).
 template <typename T, typename Reduce>
 static int launch_fast_splitk(GemmArgs g, int splits, int64_t ksteps, int bk, hipStream_t s, const Reduce& reduce) {
-  if (describe_only("dma", 4, 128, 128, splits)) return 0;
-  const size_t bytes = (size_t)splits * g.m * g.n * sizeof(float);
+  constexpr int kTile = 128;
+  g.k_chunk = (int)ceil_div(ksteps, splits) * bk;
+  const int used = (int)ceil_div(g.k, g.k_chunk);  // slices that actually hold part of K: what is launched
+  if (describe_only("dma", 4, kTile, kTile, used)) return 0;
+  const size_t bytes = (size_t)used * g.m * g.n * sizeof(float);
   float* ws = nullptr;
   {
     const int rc = splitk_workspace(bytes, s, &ws);
     if (rc != 0) return rc;
   }
-  g.k_chunk = (int)ceil_div(ksteps, splits) * bk;
-  const int used = (int)ceil_div(g.k, g.k_chunk);
-  g.tiles_m = (g.m + 127) / 128;
-  g.tiles_n = (g.n + 127) / 128;
+  g.tiles_m = (g.m + kTile - 1) / kTile;
+  g.tiles_n = (g.n + kTile - 1) / kTile;
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
   const bool vec = g.n % 4 == 0;
   EpiPartial part{ws, (int64_t)g.m * g.n, g.n, vec};
-  constexpr int LDS = fast_lds_bytes<128, 128, 2, 2>();
-  auto kern = gemm_fast_kernel<T, 128, 128, 2, 2, 2, EpiPartial>;
+  constexpr int LDS = fast_lds_bytes<kTile, kTile, 2, 2>();
+  auto kern = gemm_fast_kernel<T, kTile, kTile, 2, 2, 2, EpiPartial>;
   {
     const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
     if (rc != 0) return rc;

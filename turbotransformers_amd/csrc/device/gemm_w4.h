@@ -171,7 +171,7 @@ constexpr int kW4Threads = 256;
 constexpr int kW4Block = 16;
 
 // Epilogues whose output is one row-major matrix: base address and leading dimension, so that the kernel can
-// store through a buffer resource (32-bit offsets, rows past M dropped by the hardware's range check).
+// store through a buffer resource (32-bit offsets; rows past M are predicated off by the kernel itself).
 template <typename Epi>
 struct LinearDest : std::false_type {
   static __device__ __forceinline__ void* base(const Epi&) { return nullptr; }
@@ -297,7 +297,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, bs + (i - A_LOADS) * 1024, 16, vob[i - A_LOADS], b_soff + dma_k * kRowBytes, 0, 0);
     }
   };
-  // the output matrix of a linear epilogue: rows at and past M lie outside the resource and their stores are dropped
+  // the output matrix of a linear epilogue (the resource ends at row M; the stores are predicated on the row as well)
   const uint32_t ldc_bytes = (uint32_t)LinearDest<Epi>::ldc(epi) * (uint32_t)sizeof(T);
   const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(LinearDest<Epi>::base(epi), 0, (int)min((int64_t)g.m * ldc_bytes, (int64_t)0x7fffffff), 0x00020000);
   auto store_c = [&](Quad x, uint32_t voff, uint32_t soff) __attribute__((always_inline)) {
@@ -537,7 +537,9 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
             const uint32_t soff = (uint32_t)row0 * ldc_bytes + (uint32_t)(n0 + wn0) * (uint32_t)sizeof(T);
 #pragma unroll
             for (int pass = 0; pass < PASSES; ++pass)
-              if (whole_width || n0 + wn0 + st_col[pass] < n_lim)
+              // rows at and past M are skipped here: the scalar offset of a buffer store takes no part in the
+              // resource's range check, so the check alone would not drop a row group that lies wholly past M
+              if ((whole_rows || row0 + st_row[pass] < m_lim) && (whole_width || n0 + wn0 + st_col[pass] < n_lim))
                 store_c(landed[pass], (uint32_t)st_row[pass] * ldc_bytes + (uint32_t)st_col[pass] * (uint32_t)sizeof(T), soff);
           } else {
             const int64_t block_part = epi.row_part(min(row0, m_lim - 1));  // uniform
@@ -718,10 +720,9 @@ constexpr TileConfig kW4Tile256{256, 256, 1, 1.10f};
 template <typename T, typename Epi>
 static bool w4_wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) {
   if (!epi.vec || !w4_eligible<T>(g, batch, aligned)) return false;
-  if (const char* force = std::getenv("TTMI_LARGE_TILE")) {
-    if (force[0] == '0') return false;
-    if (force[0] == '1') return true;
-  }
+  const int force = kernel_switch(kSwitchLargeTile);
+  if (force == 0) return false;
+  if (force == 1) return true;
   double other = 0;
   (void)pick_tile(g.m, g.n, batch, &other);
   const double mine = LinearDest<Epi>::value ? std::min(tile_cost(kW4Tile192, g.m, g.n, batch), tile_cost(kW4Tile256, g.m, g.n, batch))
@@ -773,10 +774,9 @@ struct LargeTileKernel<T, EpiQkvSplit<T, false>, typename std::enable_if<sizeof(
     // eight rows of a transposed V lie in at most two sequences: what the kernel's element-wise store assumes
     // (and steps from one sequence to the next with a 32-bit element offset)
     if (epi.v_pitch > 0 && (epi.seq < 8 || (int64_t)epi.hidden * epi.v_pitch >= (1ll << 31))) return false;
-    if (const char* force = std::getenv("TTMI_LARGE_TILE")) {
-      if (force[0] == '0') return false;
-      if (force[0] == '1') return true;
-    }
+    const int force = kernel_switch(kSwitchLargeTile);
+    if (force == 0) return false;
+    if (force == 1) return true;
     double other = 0;
     (void)pick_tile(g.m, g.n, batch, &other);
     return cost(g, epi, batch) < other;

@@ -2,9 +2,31 @@
 // error plumbing shared by every kernel file.
 #include "common.h"
 
+#include <atomic>
+#include <cstdlib>
 #include <cstring>
 
 namespace ttmi {
+
+namespace {
+const char* const kSwitchNames[kNumKernelSwitches] = {"TTMI_LARGE_TILE", "TTMI_WAVE_KERNEL", "TTMI_ATTENTION_WAVES",
+                                                       "TTMI_STATIC_SCRATCH_LIMIT"};
+struct KernelSwitches {
+  std::atomic<int> value[kNumKernelSwitches];
+  KernelSwitches() {
+    for (int i = 0; i < kNumKernelSwitches; ++i) {
+      const char* text = std::getenv(kSwitchNames[i]);
+      value[i].store(text != nullptr && text[0] != 0 ? std::atoi(text) : kSwitchUnset, std::memory_order_relaxed);
+    }
+  }
+};
+KernelSwitches& kernel_switches() {
+  static KernelSwitches s;  // the environment is read here, once
+  return s;
+}
+}  // namespace
+
+int kernel_switch(KernelSwitch which) { return kernel_switches().value[which].load(std::memory_order_relaxed); }
 
 static thread_local std::string g_last_error;
 
@@ -47,6 +69,17 @@ using namespace ttmi;
 extern "C" {
 
 const char* ttmi_last_error(void) { return g_last_error.c_str(); }
+
+int ttmi_set_kernel_switch(const char* name, int value) {
+  TTMI_REQUIRE(name != nullptr, "switch name is null");
+  for (int i = 0; i < kNumKernelSwitches; ++i) {
+    if (std::strcmp(name, kSwitchNames[i]) == 0) {
+      kernel_switches().value[i].store(value, std::memory_order_relaxed);
+      return 0;
+    }
+  }
+  return fail(TTMI_EINVAL, std::string("unknown kernel switch ") + name);
+}
 
 int ttmi_device_count(int* count) {
   TTMI_REQUIRE(count != nullptr, "count is null");

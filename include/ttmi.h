@@ -48,7 +48,8 @@ enum ttmi_epilogue {
   TTMI_EPI_BIAS_ACT = 2,      /* C = act(acc + bias[n])             (AddBiasAct fused)    */
   TTMI_EPI_BIAS_RESIDUAL = 3, /* C = acc + bias[n] + residual[m,n]  (pre-LayerNorm sum)   */
   TTMI_EPI_QKV_SPLIT = 4,     /* acc + bias -> q,k,v [B,h,S,d]      (SplitAddBiasTranspose fused) */
-  TTMI_EPI_QKV_SPLIT_PAD = 5  /* packed rows -> zero-padded q,k,v [B,h,maxS,d]            */
+  TTMI_EPI_QKV_SPLIT_PAD = 5, /* packed rows -> zero-padded q,k,v [B,h,maxS,d]            */
+  TTMI_EPI_F32_OUT = 6        /* C_f32 = acc (+ bias[n] if given): c is float* whatever dtype */
 };
 
 /* ------------------------------------------------------------------ runtime ---------- */
@@ -126,6 +127,15 @@ TTMI_API int ttmi_add_bias_layer_norm_residual32(void* out, const float* residua
                                                  const void* gamma, const void* beta, float* out_f32, int64_t m,
                                                  int64_t n, float eps, int dtype, void* stream);
 
+/* The same with the product itself in fp32: product_out_f32[m,n] holds a[m,k] . w[n,k]^T as the GEMM accumulated it
+ * (ttmi_gemm_fused with TTMI_EPI_F32_OUT) and is overwritten with the unrounded result,
+ *   y = LN(product_out_f32 + residual_f32 + bias);  out = round(y);  product_out_f32 = y.
+ * product_out_f32 must not alias residual_f32.  No counterpart in the reference (fp32-only, where this is plain
+ * AddBiasLayerNorm, layers/kernels/layer_norm.cpp:99-180). */
+TTMI_API int ttmi_add_bias_layer_norm_product32(void* out, const float* residual_f32, const void* bias,
+                                                const void* gamma, const void* beta, float* product_out_f32,
+                                                int64_t m, int64_t n, float eps, int dtype, void* stream);
+
 /* The dense projection and AddBiasLayerNorm that close both halves of an encoder layer, as one call:
  *   out[m,n] = LN(a[m,k] . w[n,k]^T + bias + residual)
  * (BertOutput, layers/bert_output.cpp:41-60; the attention output, layers/multi_headed_attention.cpp:359-371;
@@ -133,7 +143,9 @@ TTMI_API int ttmi_add_bias_layer_norm_residual32(void* out, const float* residua
  * fill the chip, normalise inside the kernel that sums the K slices; larger ones run ttmi_gemm followed by
  * ttmi_add_bias_layer_norm.  Either `residual` (same dtype as out) or the pair residual_f32 / out_f32 (the
  * fp32 residual stream of ttmi_add_bias_layer_norm_residual32, which may alias each other) is given; the
- * unused ones are NULL.  `out` must not alias `residual` or `a` (large problems store the bare product to `out`
+ * unused ones are NULL.  With the fp32 pair and out_f32 != residual_f32, 16-bit products of large problems are kept
+ * in fp32 between the GEMM and the LayerNorm (in out_f32), as the K-sliced path does for small ones; when the two
+ * alias, the product of a large problem passes through `out` in the 16-bit type.  `out` must not alias `residual` or `a` (large problems store the bare product to `out`
  * before the residual is read); a call that passes the same buffer is refused.  a, w, out are densely packed
  * (lda = ldb = k, ldc = n). */
 TTMI_API int ttmi_gemm_bias_layer_norm(const void* a, const void* w, void* out, const void* residual,
@@ -330,6 +342,8 @@ typedef struct ttmi_epilogue_args {
  *                    (layers/bert_output.cpp:47-51, layers/multi_headed_attention.cpp:359-371)
  *   QKV_SPLIT[_PAD]= MatMul + SplitAddBiasTransposeForScore[Pad]
  *                    (layers/multi_headed_attention.cpp:199-203, ..._smart_batch.cpp:212-217)
+ *   F32_OUT        = MatMul whose result leaves in fp32 (c is float*, ldc in floats; bias optional): what a 16-bit
+ *                    model hands to AddBiasLayerNorm without rounding it first
  * B is always [N,K] here (weights are repacked K-contiguous at construction).
  * For the QKV forms `c` may be NULL. */
 TTMI_API int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,

@@ -256,10 +256,46 @@ def test_gemm_bias_layer_norm_fp32_residual(ttmi, oracle, dt, M, N, K):
     want = oracle.add_bias_layer_norm(base, res, rounded(bias, dt), rounded(gamma, dt), rounded(beta, dt))
     assert _ln_close(host(out32), want, dt)
     assert np.array_equal(host(out), rounded(host(out32), dt))
+    # with its own fp32 output buffer nothing is rounded between the accumulators and the normalisation, on the
+    # K-sliced path and on the large-problem path alike: the fp32 result is as close to the oracle as an fp32 run
+    assert _ln_close(host(out32), want, "f32")
     first = out32.clone()
     ok(ttmi.ttmi_gemm_bias_layer_norm(ptr(dA), ptr(dW), ptr(out), None, ptr(dres), *args, ptr(dres), M, N, K, 1e-12,
                                       TTMI_DTYPES[dt], stream()))
-    assert torch.equal(dres, first)
+    if M <= 128:
+        assert torch.equal(dres, first)  # K-sliced: the same kernels either way
+    else:
+        # a large problem writing over its residual has nowhere to keep an fp32 product: it passes through `out`
+        # in the 16-bit type, one more rounding
+        assert _ln_close(host(dres), want, dt)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("forced", [False, True])
+@pytest.mark.parametrize("M,N,K,with_bias", [(300, 200, 256, True), (4100, 1024, 1024, False), (2560, 768, 3072, True),
+                                             (8192, 768, 768, True), (777, 776, 384, False), (128, 768, 3072, True)])
+def test_gemm_with_fp32_output(ttmi, oracle, dt, forced, M, N, K, with_bias):
+    """TTMI_EPI_F32_OUT: 16-bit operands, the accumulators (plus an optional bias) stored as fp32.  Tile kernels of
+    every family (small tiles, K slices, the 8-wavefront DMA tiles, the one-wavefront-per-SIMD kernel with whole and
+    ragged tiles, also forced onto small shapes): the result is the fp32 product of the rounded operands, to fp32
+    accumulation error, and rows past M stay untouched."""
+    import ctypes
+    rng = np.random.default_rng(M + N + K)
+    A, W = _ab(rng, M, N, K, 1)
+    bias = rng.standard_normal(N).astype(np.float32)
+    dA, dW, db = dev(A, dt), dev(W, dt), dev(bias, dt)
+    whole = torch.full((M + 64, N), -7.0, device="cuda")
+    C = whole[:M]
+    if forced:
+        ok(ttmi.ttmi_set_kernel_switch(b"TTMI_LARGE_TILE", 1))
+    try:
+        ok(ttmi.ttmi_gemm_fused(ptr(dA), ptr(dW), ptr(C), M, N, K, K, K, N, capi.EPI_F32_OUT,
+                                ctypes.byref(_epi(bias=db) if with_bias else _epi()), TTMI_DTYPES[dt], stream()))
+    finally:
+        ok(ttmi.ttmi_set_kernel_switch(b"TTMI_LARGE_TILE", -1))
+    want = oracle.matmul(rounded(A, dt), rounded(W, dt), True) + (rounded(bias, dt) if with_bias else 0.0)
+    assert max_abs(host(C), want) <= GEMM_TOL["f32"] * max(1.0, float(np.abs(want).max()))
+    assert torch.all(whole[M:] == -7.0)
 
 
 def test_gemm_bias_layer_norm_rejects_bad_arguments(ttmi):

@@ -53,6 +53,27 @@ def test_add_bias_layer_norm_fp32_residual(ttmi, oracle, dt, m, n):
     assert max_abs(host(d_res), want) <= 1e-4
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("m,n", [(37, 768), (8, 1024), (5, 770), (300, 5000)])
+def test_add_bias_layer_norm_fp32_product(ttmi, oracle, dt, m, n):
+    """The product arrives in fp32 as well (in the buffer that receives the fp32 result): the result equals the
+    oracle on the same fp32 values to fp32 accuracy, the 16-bit output is its rounding, and a product buffer that
+    aliases the residual is refused."""
+    rng = np.random.default_rng(n + 1)
+    prod, res = rng.standard_normal((m, n), np.float32), rng.standard_normal((m, n), np.float32)
+    bias, gamma, beta = (rng.standard_normal(n).astype(np.float32) for _ in range(3))
+    d_out = torch.full((m, n), float("nan"), dtype=dev(bias, dt).dtype, device="cuda")
+    d_prod, d_res = dev(prod), dev(res)
+    vecs = (ptr(dev(bias, dt)), ptr(dev(gamma, dt)), ptr(dev(beta, dt)))
+    ok(ttmi.ttmi_add_bias_layer_norm_product32(ptr(d_out), ptr(d_res), *vecs, ptr(d_prod), m, n, 1e-12, TTMI_DTYPES[dt], stream()))
+    want = oracle.add_bias_layer_norm(prod, res, rounded(bias, dt), rounded(gamma, dt), rounded(beta, dt))
+    assert max_abs(host(d_prod), want) <= 1e-4
+    assert np.array_equal(host(d_out), rounded(host(d_prod), dt))
+    assert np.array_equal(host(d_res), res)
+    assert ttmi.ttmi_add_bias_layer_norm_product32(ptr(d_out), ptr(d_res), *vecs, ptr(d_res), m, n, 1e-12, TTMI_DTYPES[dt],
+                                                   stream()) == -1
+
+
 @pytest.mark.parametrize("n", [768, 1000, 4096])
 def test_layer_norm_of_near_constant_rows_stays_finite(ttmi, n):
     """E[x^2] - mean^2 (the reference's formula, layer_norm.cpp:144-163) cancels on a row whose spread is far below its

@@ -57,8 +57,10 @@ def test_static_scratch_fp32_residual_stream(ttmi, dt):
 
 
 def test_static_scratch_unsplit_problems_need_no_scratch(ttmi):
-    """A problem large enough to run unsplit uses no partial tiles and is accepted at any size."""
+    """A problem large enough to run unsplit uses no partial tiles and is accepted at any size (with an fp32
+    residual stream its fp32 product lives in the caller's own fp32 output buffer)."""
     _both(ttmi, "f16", 8192, 768, 768, seed=6)
+    _both(ttmi, "bf16", 8192, 1024, 1024, seed=10, fp32_residual=True)
 
 
 def test_static_scratch_refuses_what_does_not_fit(ttmi):

@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(_PKG, "lib", "libttmi.so")
 F32, F16, BF16, I8, I32, I64 = range(6)
 ACT_GELU, ACT_TANH, ACT_RELU = range(3)
 H2D, D2H, D2D = range(3)
-EPI_NONE, EPI_BIAS, EPI_BIAS_ACT, EPI_BIAS_RESIDUAL, EPI_QKV_SPLIT, EPI_QKV_SPLIT_PAD = range(6)
+EPI_NONE, EPI_BIAS, EPI_BIAS_ACT, EPI_BIAS_RESIDUAL, EPI_QKV_SPLIT, EPI_QKV_SPLIT_PAD, EPI_F32_OUT = range(7)
 QUANT_SCALE_FLOATS = 514  # TTMI_QUANT_SCALE_FLOATS
 
 

@@ -76,6 +76,15 @@ static int gemm_bias_layer_norm_impl(const void* a, const void* w, void* out, co
     }
   });
   // Large problems: the GEMM kernel's own tiles cover the chip; LayerNorm follows as its own pass.
+  // With an fp32 residual stream and room for it, the product stays in fp32 too: the GEMM stores its accumulators to
+  // out_f32 and the LayerNorm pass reads them there, so that (as in the K-sliced path above) nothing is rounded
+  // between the matrix pipe and the normalisation.
+  if (residual_f32 != nullptr && out_f32 != residual_f32 && dtype != TTMI_F32) {
+    ttmi_epilogue_args f32_args{};
+    const int rc = ttmi_gemm_fused(a, w, out_f32, m, n, k, k, k, n, TTMI_EPI_F32_OUT, &f32_args, dtype, stream);
+    if (rc != 0) return rc;
+    return ttmi_add_bias_layer_norm_product32(out, residual_f32, bias, gamma, beta, out_f32, m, n, eps, dtype, stream);
+  }
   const int rc = ttmi_gemm(a, w, out, m, n, k, k, k, n, 1, 1.f, 0.f, dtype, stream);
   if (rc != 0) return rc;
   if (residual_f32 != nullptr)
@@ -160,6 +169,11 @@ int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, int64_t n,
           return (launch_gemm<T, false>(g, epi, 1, aligned, s));
         }
         return fail(TTMI_EINVAL, "unknown activation");
+      }
+      case TTMI_EPI_F32_OUT: {
+        TTMI_REQUIRE(c && ldc >= n, "F32_OUT epilogue needs c");
+        EpiF32<T> epi{(float*)c, (const T*)args->bias, ldc, aligned16(c) && ldc % 4 == 0 && aligned16(args->bias)};
+        return (launch_gemm<T, false>(g, epi, 1, aligned, s));
       }
       case TTMI_EPI_BIAS_RESIDUAL: {
         TTMI_REQUIRE(c && args->bias && args->residual && ldc >= n, "BIAS_RESIDUAL epilogue needs c, bias, residual");

@@ -846,6 +846,32 @@ struct EpiPartial {
   }
 };
 
+// acc (+ bias) -> an fp32 matrix whatever the operand type: a product that feeds a LayerNorm keeps the precision of
+// its accumulators (with bfloat16 storage the rounding of that product to 8 bits is the largest single contribution
+// to the deviation of a deep encoder from fp32 arithmetic).
+template <typename T>
+struct EpiF32 {
+  using Acc = float;
+  float* c;
+  const T* bias;  // may be null
+  int64_t ldc;
+  bool vec;
+  __device__ __forceinline__ const T* bias_ptr() const { return bias; }
+  __device__ __forceinline__ float finish(float x) const { return x; }
+  __device__ __forceinline__ void store8(int, int m, int n, float (&v)[8], int valid) const {
+    float* p = c + (int64_t)m * ldc + n;
+    if (vec && valid == 8) {
+      store_row8<float>(p, v);
+    } else {
+      for (int j = 0; j < valid; ++j) p[j] = v[j];
+    }
+  }
+};
+template <typename Epi>
+struct StoresF32 : std::false_type {};
+template <typename T>
+struct StoresF32<EpiF32<T>> : std::true_type {};
+
 template <typename Epi>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int m, int n, bool vec,
                                                             const Epi epi) {

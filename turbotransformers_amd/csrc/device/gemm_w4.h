@@ -486,7 +486,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       // epilogues that scatter (the QKV split): the column part of a lane's destinations, once per tile
       T* col_ptr[PASSES];
       bool block_in_one_sequence = false;  // uniform: the rows of a group share their batch index
-      if constexpr (!LinearDest<Epi>::value) {
+      if constexpr (!LinearDest<Epi>::value && !StoresF32<Epi>::value) {
         block_in_one_sequence = epi.rows_share_sequence(GROUP);
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
@@ -495,6 +495,9 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
         }
       }
       Quad landed[PASSES];  // first-class vectors: arrays of a struct type may end up in scratch memory
+      // The matrix instructions are inline asm, so the compiler's hazard recogniser does not see that the accumulator
+      // reads below depend on them: wait out the longest write-to-read distance of the matrix pipe here.
+      asm volatile("s_nop 15\n\ts_nop 15");
 #pragma unroll
       for (int i = 0; i <= GROUPS; ++i) {
         Quad packed[NV];
@@ -524,16 +527,30 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
                 bv[v % NBV].add_to(out);
               }
             }
-            T rounded[8];
+            if constexpr (StoresF32<Epi>::value) {
+              // fp32 output: the lane's eight columns are 32 contiguous bytes of one row, and the four lanes that share
+              // a row cover 128 contiguous bytes between them: stored as they lie, no trip through the strip
+              const int m = m0 + wm0 + i * GROUP + (MF == 32 ? lrow : 16 * (v / (CB / 2)) + lrow);
+              const int ncol = n0 + wn0 + unit_chunk(v) * 8;
+              if ((whole_rows || m < m_lim) && (whole_width || ncol < n_lim)) {
+                float* dst = epi.c + (int64_t)m * epi.ldc + ncol;
+                *reinterpret_cast<floatx4*>(dst) = floatx4{out[0], out[1], out[2], out[3]};
+                *reinterpret_cast<floatx4*>(dst + 4) = floatx4{out[4], out[5], out[6], out[7]};
+              }
+              packed[v] = Quad{0, 0, 0, 0};
+            } else {
+              T rounded[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) rounded[e] = from_float<T>(epi.finish(out[e]));
-            packed[v] = __builtin_bit_cast(Quad, pack_chunk(rounded));
+              for (int e = 0; e < 8; ++e) rounded[e] = from_float<T>(epi.finish(out[e]));
+              packed[v] = __builtin_bit_cast(Quad, pack_chunk(rounded));
+            }
           }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (i > 0) {
+        if (i > 0 && !StoresF32<Epi>::value) {
           const int row0 = m0 + wm0 + (i - 1) * GROUP;
-          if constexpr (LinearDest<Epi>::value) {
+          if constexpr (StoresF32<Epi>::value) {
+          } else if constexpr (LinearDest<Epi>::value) {
             const uint32_t soff = (uint32_t)row0 * ldc_bytes + (uint32_t)(n0 + wn0) * (uint32_t)sizeof(T);
 #pragma unroll
             for (int pass = 0; pass < PASSES; ++pass)
@@ -552,7 +569,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
           }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (i < GROUPS) {
+        if (i < GROUPS && !StoresF32<Epi>::value) {
           // same wavefront, LDS operations complete in order: no barrier between the writes and the reads
 #pragma unroll
           for (int v = 0; v < NV; ++v) strip_write(strip_lds + (uint32_t)wr_off[v], packed[v]);
@@ -582,6 +599,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
         const bool rows_whole = m0 + BM <= m_lim && epi.seq % 8 == 0;  // uniform: every group of eight is one store
         T* const vt_base = epi.vt_col_part((uint32_t)min(n0 + wn0 + rd_col, n_lim - 1));
         Quad vt_landed[VP];
+        asm volatile("s_nop 15\n\ts_nop 15");  // as in the row path: the accumulator reads follow inline-asm matrix instructions
 #pragma unroll
         for (int u = 0; u <= UNITS; ++u) {
           Quad piece[4];
@@ -725,7 +743,7 @@ static bool w4_wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned
   if (force == 1) return true;
   double other = 0;
   (void)pick_tile(g.m, g.n, batch, &other);
-  const double mine = LinearDest<Epi>::value ? std::min(tile_cost(kW4Tile192, g.m, g.n, batch), tile_cost(kW4Tile256, g.m, g.n, batch))
+  const double mine = (LinearDest<Epi>::value || StoresF32<Epi>::value) ? std::min(tile_cost(kW4Tile192, g.m, g.n, batch), tile_cost(kW4Tile256, g.m, g.n, batch))
                                              : tile_cost(kW4Tile192, g.m, g.n, batch);
   return mine < other;
 }
@@ -784,6 +802,16 @@ struct LargeTileKernel<T, EpiQkvSplit<T, false>, typename std::enable_if<sizeof(
   static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) {
     if (fits256(g, epi) && tile_cost(kTile256, g.m, g.n, 1) < cost192(g, epi, 1)) return launch_w4<T, 256>(g, epi, s);
     return launch_w4<T, 192>(g, epi, s, split_run(g, epi) ? 2 * epi.hidden : 0);
+  }
+};
+// fp32 output of a 16-bit product (the projections in front of a LayerNorm in bfloat16 models).
+template <typename T>
+struct LargeTileKernel<T, EpiF32<T>, typename std::enable_if<sizeof(T) == 2>::type> {
+  using Epi = EpiF32<T>;
+  static bool wanted(const GemmArgs& g, const Epi& epi, int batch, bool aligned) { return w4_wanted<T>(g, epi, batch, aligned); }
+  static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) {
+    if (tile_cost(kW4Tile256, g.m, g.n, 1) < tile_cost(kW4Tile192, g.m, g.n, 1)) return launch_w4<T, 256>(g, epi, s);
+    return launch_w4<T, 192>(g, epi, s);
   }
 };
 template <typename T>

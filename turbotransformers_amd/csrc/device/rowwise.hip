@@ -15,10 +15,12 @@ constexpr int kBlock = 256;
 // x = out (+ input + bias); mean = sum(x)/n; var = sum(x*x)/n - mean^2;
 // out = beta + gamma * (x - mean) * rsqrt(var + eps)      (layer_norm.cpp:144-163)
 //
-// RES32: the residual is read from an fp32 copy (`res32`) instead of `input`, and the result is
+// RES32 = 1: the residual is read from an fp32 copy (`res32`) instead of `input`, and the result is
 // also written unrounded to `out32`.  With 16-bit storage this keeps the residual stream of the
 // encoder in fp32 -- only GEMM operands are rounded -- at the cost of 12 instead of 6 bytes/element.
-template <typename T, int VEC, int G, int ITERS, bool ADD, bool RES32>
+// RES32 = 2: in addition the product itself arrives unrounded, in `out32` (which this kernel then overwrites with
+// the result, element by element, each by the thread that read it); `out` is only written: 14 bytes/element.
+template <typename T, int VEC, int G, int ITERS, bool ADD, int RES32>
 __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, const T* __restrict__ input,
                                                           const T* __restrict__ bias,
                                                           const T* __restrict__ gamma,
@@ -37,8 +39,13 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
   for (int it = 0; it < ITERS; ++it) {
     const int col = (it * G + lane) * VEC;
     if (row_ok && col < n) {
-      Vec<T, VEC> o = load_vec<T, VEC>(orow + col);
-      if (ADD && RES32) {
+      Vec<T, VEC> o;
+      if (RES32 != 2) o = load_vec<T, VEC>(orow + col);
+      if (ADD && RES32 == 2) {
+        Vec<T, VEC> b = load_vec<T, VEC>(bias + col);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[it][j] = out32[row * n + col + j] + res32[row * n + col + j] + to_float(b.v[j]);
+      } else if (ADD && RES32) {
         Vec<T, VEC> b = load_vec<T, VEC>(bias + col);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) x[it][j] = to_float(o.v[j]) + res32[row * n + col + j] + to_float(b.v[j]);
@@ -75,7 +82,8 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
       Vec<T, VEC> o;
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        const float y = to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean);
+        float y = to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean);
+        if (RES32) asm volatile("" : "+v"(y));  // out is the rounding of the fp32 value, not of the exact multiply-add
         o.v[j] = from_float<T>(y);
         if (RES32) out32[row * n + col + j] = y;
       }
@@ -85,7 +93,7 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
 }
 
 // Fallback: one block per row, any n; the row is re-read from L2 for the second pass.
-template <typename T, bool ADD, bool RES32>
+template <typename T, bool ADD, int RES32>
 __global__ __launch_bounds__(kBlock) void layer_norm_block(T* __restrict__ out, const T* __restrict__ input,
                                                            const T* __restrict__ bias,
                                                            const T* __restrict__ gamma,
@@ -98,7 +106,7 @@ __global__ __launch_bounds__(kBlock) void layer_norm_block(T* __restrict__ out, 
   const float* rrow = RES32 ? res32 + row * n : nullptr;
   float sum = 0.f, sumsq = 0.f;
   for (int c = threadIdx.x; c < n; c += kBlock) {
-    float x = to_float(orow[c]);
+    float x = RES32 == 2 ? out32[row * n + c] : to_float(orow[c]);
     if (ADD) x = x + (RES32 ? rrow[c] : to_float(irow[c])) + to_float(bias[c]);
     sum += x;
     sumsq += x * x;
@@ -121,15 +129,18 @@ __global__ __launch_bounds__(kBlock) void layer_norm_block(T* __restrict__ out, 
   const float var = fmaxf(sumsq / (float)n - mean * mean, 0.f);  // cancellation on a near-constant row must not go negative
   const float rstd = 1.0f / sqrtf(var + eps);
   for (int c = threadIdx.x; c < n; c += kBlock) {
-    float x = to_float(orow[c]);
+    float x = RES32 == 2 ? out32[row * n + c] : to_float(orow[c]);
     if (ADD) x = x + (RES32 ? rrow[c] : to_float(irow[c])) + to_float(bias[c]);
-    const float y = to_float(beta[c]) + to_float(gamma[c]) * rstd * (x - mean);
+    float y = to_float(beta[c]) + to_float(gamma[c]) * rstd * (x - mean);
+    // the 16-bit output is the rounding of the fp32 one: keep the compiler from folding the conversion into the
+    // multiply-add (a mixed-precision fma rounds the exact result once, not the fp32 value)
+    if (RES32) asm volatile("" : "+v"(y));
     orow[c] = from_float<T>(y);
     if (RES32) out32[row * n + c] = y;
   }
 }
 
-template <typename T, int VEC, int G, int ITERS, bool ADD, bool RES32>
+template <typename T, int VEC, int G, int ITERS, bool ADD, int RES32>
 static int launch_ln_rows(T* out, const T* input, const T* bias, const T* gamma, const T* beta, int64_t m,
                           int n, float eps, const float* res32, float* out32, hipStream_t s) {
   constexpr int ROWS = kBlock / G;
@@ -139,7 +150,7 @@ static int launch_ln_rows(T* out, const T* input, const T* bias, const T* gamma,
   return launch_status("layer_norm_rows");
 }
 
-template <typename T, bool ADD, bool RES32 = false>
+template <typename T, bool ADD, int RES32 = 0>
 static int layer_norm_dispatch(T* out, const T* input, const T* bias, const T* gamma, const T* beta,
                                int64_t m, int64_t n, float eps, hipStream_t s, const float* res32 = nullptr,
                                float* out32 = nullptr) {
@@ -402,10 +413,23 @@ int ttmi_add_bias_layer_norm_residual32(void* out, const float* residual_f32, co
                                         int dtype, void* stream) {
   TTMI_REQUIRE(out && residual_f32 && bias && gamma && beta && out_f32, "null tensor");
   TTMI_REQUIRE(m >= 0 && n >= 0 && n < (1ll << 31), "bad shape");
-  TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, true, true>((T*)out, nullptr, (const T*)bias,
+  TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, true, 1>((T*)out, nullptr, (const T*)bias,
                                                                             (const T*)gamma, (const T*)beta, m, n,
                                                                             eps, (hipStream_t)stream, residual_f32,
                                                                             out_f32)));
+  return 0;
+}
+
+int ttmi_add_bias_layer_norm_product32(void* out, const float* residual_f32, const void* bias, const void* gamma,
+                                       const void* beta, float* product_out_f32, int64_t m, int64_t n, float eps,
+                                       int dtype, void* stream) {
+  TTMI_REQUIRE(out && residual_f32 && bias && gamma && beta && product_out_f32, "null tensor");
+  TTMI_REQUIRE(residual_f32 != product_out_f32, "the fp32 product must not alias the residual");
+  TTMI_REQUIRE(m >= 0 && n >= 0 && n < (1ll << 31), "bad shape");
+  TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, true, 2>((T*)out, nullptr, (const T*)bias,
+                                                                         (const T*)gamma, (const T*)beta, m, n, eps,
+                                                                         (hipStream_t)stream, residual_f32,
+                                                                         product_out_f32)));
   return 0;
 }
 

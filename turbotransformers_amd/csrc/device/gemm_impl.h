@@ -439,18 +439,13 @@ struct EpiDequant {
   int64_t ldc;
   bool vec;
   int act;  // ttmi_act, applied after the bias
-  __device__ __forceinline__ const float* bias_ptr() const { return nullptr; }  // added after scaling, below
+  __device__ __forceinline__ const float* bias_ptr() const { return bias; }
+  __device__ __forceinline__ bool has_bias() const { return bias != nullptr; }
+  // v: the bit patterns of the dequantised values (dequantise() below, applied in accumulator layout)
   __device__ __forceinline__ void store8(int, int m, int n, int (&v)[8], int valid) const {
-    const float sx = act_scale[0];
     float r[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      r[j] = 0.f;
-      if (j < valid) {
-        r[j] = (float)v[j] * sx * w_scale[n + j];
-        if (bias) r[j] += bias[n + j];
-      }
-    }
+    for (int j = 0; j < 8; ++j) r[j] = __builtin_bit_cast(float, v[j]);
     if (act == TTMI_ACT_GELU) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) r[j] = apply_act<TTMI_ACT_GELU>(r[j]);
@@ -478,19 +473,45 @@ struct EpiDequantQkvSplit {
   EpiQkvSplit<float, false> split;  // its bias is added here, after the scaling
   const float* act_scale;           // device scalar
   const float* w_scale;             // [N]
-  __device__ __forceinline__ const float* bias_ptr() const { return nullptr; }
+  __device__ __forceinline__ const float* bias_ptr() const { return split.bias; }
+  __device__ __forceinline__ bool has_bias() const { return true; }
   __device__ __forceinline__ void store8(int z, int m, int n, int (&v)[8], int valid) const {
-#pragma clang fp contract(off)  // the bias is added to the ROUNDED product, as the separate kernel does
-    const float sx = act_scale[0];
     float r[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float scaled = (float)v[j] * sx * w_scale[j < valid ? n + j : n];
-      r[j] = scaled + split.bias[j < valid ? n + j : n];
-    }
+    for (int j = 0; j < 8; ++j) r[j] = __builtin_bit_cast(float, v[j]);
     split.store8(z, m, n, r, valid);
   }
 };
+
+// The dequantising epilogues scale in ACCUMULATOR layout, where a lane owns one column per 32 x 32 block: the
+// activation scale and the lane's few weight scales and biases are fetched once per tile, next to the bias columns
+// of the other epilogues (fetched per stored row segment they were 17 dependent loads in front of every store).
+// float(acc) * act_scale * w_scale[n], then + bias[n], each product and the sum rounded: the operation order of
+// dequant_bias_kernel, so that the fused and the two-kernel form give the same bits.
+template <typename Epi>
+struct Dequantises : std::false_type {};
+template <>
+struct Dequantises<EpiDequant> : std::true_type {};
+template <>
+struct Dequantises<EpiDequantQkvSplit> : std::true_type {};
+__device__ __forceinline__ float dequantise(int acc, float act_scale, float w_scale, float bias, bool has_bias) {
+#pragma clang fp contract(off)
+  float r = (float)acc * act_scale * w_scale;
+  if (has_bias) r = r + bias;
+  return r;
+}
+// sj[0..TN) = weight scales of the lane's columns, sj[TN] = activation scale; untouched for other epilogues
+template <int TN, typename Epi>
+__device__ __forceinline__ void load_dequant_columns(const Epi& epi, int n_first, int n_limit, float (&sj)[TN + 1]) {
+  if constexpr (Dequantises<Epi>::value) {
+    sj[TN] = epi.act_scale[0];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n_first + j * 32;
+      sj[j] = n < n_limit ? epi.w_scale[n] : 0.f;
+    }
+  }
+}
 
 // -------------------------------------------------------------------------- kernel ------
 // LDS rows are 128 bytes and the LDS has 64 four-byte banks (256 bytes per bank cycle): rows r and
@@ -512,9 +533,9 @@ struct HasColumnPass<EpiQkvSplit<T, PAD>> : std::true_type {};
 // columns from first_column_of_pass() on read back column-major instead: 8 rows of one column
 // per lane, four adjacent lanes covering 32 consecutive rows = 64 contiguous output bytes.
 template <typename T, int TM, int TN, int NT, int LDS_BYTES, typename Epi>
-__device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], const float (&bj)[TN], char* smem,
-                                           const Epi& epi, const GemmArgs& g, int z, int wave_m0, int wave_n0, int lane,
-                                           int wave) {
+__device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], const float (&bj)[TN], const float (&sj)[TN + 1],
+                                           char* smem, const Epi& epi, const GemmArgs& g, int z, int wave_m0, int wave_n0,
+                                           int lane, int wave) {
   using AccScalar = typename Mma<T>::AccScalar;
   constexpr int W = TN * 32;             // strip width (columns)
   constexpr int LDW = W + 4;             // padded pitch in words: rows stay 16-byte aligned
@@ -528,8 +549,14 @@ __device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], 
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e)
-        stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = acc[i][j][e] + (AccScalar)bj[j];
+      for (int e = 0; e < 16; ++e) {
+        AccScalar staged;
+        if constexpr (Dequantises<Epi>::value)
+          staged = __builtin_bit_cast(AccScalar, dequantise(acc[i][j][e], sj[TN], sj[j], bj[j], epi.has_bias()));
+        else
+          staged = acc[i][j][e] + (AccScalar)bj[j];
+        stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = staged;
+      }
     bool row_pass = true;
     if constexpr (HasColumnPass<Epi>::value) {
       if (epi.column_pass()) {
@@ -750,9 +777,10 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
     }
   }
 
-  float bj[TN];
+  float bj[TN], sj[TN + 1];
   load_bias_columns<TN>(epi, n0 + wn0 + lrow, g.n, bj);
-  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, bj, smem, epi, g, z_epi, m0 + wm0, n0 + wn0, lane, wave);
+  load_dequant_columns<TN>(epi, n0 + wn0 + lrow, g.n, sj);
+  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, bj, sj, smem, epi, g, z_epi, m0 + wm0, n0 + wn0, lane, wave);
 }
 
 // ------------------------------------------------------------------ wavefront kernel -----
@@ -791,8 +819,9 @@ __global__ __launch_bounds__(kWave) void gemm_wave_kernel(const GemmArgs g, cons
   const T* pa = reinterpret_cast<const T*>(g.a) + (int64_t)min(m0 + lrow, g.m - 1) * g.lda + k_lo + lhalf * 8;
   const T* pb = reinterpret_cast<const T*>(g.b) + (int64_t)min(n0 + lrow, g.n - 1) * g.ldb + k_lo + lhalf * 8;
 
-  float bj[1];
+  float bj[1], sj[2];
   load_bias_columns<1>(epi, n0 + lrow, g.n, bj);
+  load_dequant_columns<1>(epi, n0 + lrow, g.n, sj);
   Acc acc[1][1];
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[0][0][e] = 0;
@@ -820,7 +849,7 @@ __global__ __launch_bounds__(kWave) void gemm_wave_kernel(const GemmArgs g, cons
       }
     }
   }
-  store_tile<T, 1, 1, kWave, STRIP>(acc, bj, strip, epi, g, z_epi, m0, n0, lane, 0);
+  store_tile<T, 1, 1, kWave, STRIP>(acc, bj, sj, strip, epi, g, z_epi, m0, n0, lane, 0);
 }
 
 // ---------------------------------------------------------------------------- split-K -----
@@ -1150,8 +1179,9 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
     int tile_m, tile_n;
     tile_coords(logical, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    float bj[TN];
+    float bj[TN], sj[TN + 1];
     load_bias_columns<TN>(epi, n0 + wn0 + lrow, g.n, bj);
+    load_dequant_columns<TN>(epi, n0 + wn0 + lrow, g.n, sj);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1207,8 +1237,8 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
       // stores, one round trip per strip; after this wait the strips' stores are issued back to back.
       __builtin_amdgcn_s_waitcnt(0x0F70);
     }
-    store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN, NS>() - STAGE>(acc, bj, smem + STAGE, epi, g, z_epi, m0 + wm0,
-                                                                         n0 + wn0, lane, wave);
+    store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN, NS>() - STAGE>(acc, bj, sj, smem + STAGE, epi, g, z_epi, m0 + wm0,
+                                                                             n0 + wn0, lane, wave);
     if (next >= xcd_end) break;
     logical = next;
   }

@@ -76,9 +76,10 @@ __global__ __launch_bounds__(256) void dequant_bias_kernel(const int32_t* __rest
   int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (; i < total; i += stride) {
+#pragma clang fp contract(off)  // each product and the sum rounded, as the int8 GEMM's own dequantising store does
     const int c = (int)(i % n);
     float v = (float)acc[i] * sx * w_scale[c];
-    if (bias) v += bias[c];
+    if (bias) v = v + bias[c];
     out[i] = v;
   }
 }

@@ -88,13 +88,17 @@ def test_fused_epilogues_small_m_long_k(ttmi, oracle, dt):
     assert max_abs(host(C), base + rounded(bias, dt) + rounded(res, dt)) <= GEMM_TOL[dt] * 3
 
 
-@pytest.fixture
-def large_tile_forced(ttmi):
+@pytest.fixture(params=["3 A stages", "2 A stages"])
+def large_tile_forced(request, ttmi):
     """Switch TTMI_LARGE_TILE = 1 sends every eligible problem to the one-wavefront-per-SIMD kernel whatever its
-    size (set through the C ABI: the library reads its environment variables only once)."""
+    size (set through the C ABI: the library reads its environment variables only once).  Both forms of its K loop:
+    three LDS stages for the A operand where they fit (192-wide tiles, row-major outputs), and two everywhere."""
     ok(ttmi.ttmi_set_kernel_switch(b"TTMI_LARGE_TILE", 1))
+    if request.param == "2 A stages":
+        ok(ttmi.ttmi_set_kernel_switch(b"TTMI_W4_A_STAGES", 2))
     yield
     ok(ttmi.ttmi_set_kernel_switch(b"TTMI_LARGE_TILE", -1))
+    ok(ttmi.ttmi_set_kernel_switch(b"TTMI_W4_A_STAGES", -1))
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])

@@ -49,6 +49,9 @@ struct MmaBlock<f16, 32> {
   static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void run_zero(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), Acc{}, 0, 0, 0);
+  }
 };
 template <>
 struct MmaBlock<bf16, 32> {
@@ -56,12 +59,18 @@ struct MmaBlock<bf16, 32> {
   static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void run_zero(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), Acc{}, 0, 0, 0);
+  }
 };
 template <>
 struct MmaBlock<int8_t, 32> {
   using Acc = intx16;
   static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
     c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void run_zero(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), Acc{}, 0, 0, 0);
   }
 };
 template <>
@@ -73,6 +82,12 @@ struct MmaBlock<f16, 16> {
   static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(__builtin_bit_cast(halfx8, a)), "v"(__builtin_bit_cast(halfx8, b)));
   }
+  // The first product of a tile: C = A.B with the constant 0 as the addend, so the accumulator is only written.
+  // Zeroing it beforehand would cost a register write per accumulator, and (the matrix instruction being inline asm)
+  // the compiler does not know to keep the wait states between such a write and the instruction that reads it.
+  static __device__ __forceinline__ void run_zero(const Chunk& a, const Chunk& b, Acc& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(__builtin_bit_cast(halfx8, a)), "v"(__builtin_bit_cast(halfx8, b)));
+  }
 };
 template <>
 struct MmaBlock<bf16, 16> {
@@ -83,12 +98,18 @@ struct MmaBlock<bf16, 16> {
   static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(__builtin_bit_cast(bf16x8, a)), "v"(__builtin_bit_cast(bf16x8, b)));
   }
+  static __device__ __forceinline__ void run_zero(const Chunk& a, const Chunk& b, Acc& c) {  // see the fp16 form
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(__builtin_bit_cast(bf16x8, a)), "v"(__builtin_bit_cast(bf16x8, b)));
+  }
 };
 template <>
 struct MmaBlock<int8_t, 16> {
   using Acc = intx4;
   static __device__ __forceinline__ void run(const Chunk& a, const Chunk& b, Acc& c) {
     c = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void run_zero(const Chunk& a, const Chunk& b, Acc& c) {
+    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), Acc{}, 0, 0, 0);
   }
 };
 
@@ -203,15 +224,29 @@ __device__ unsigned long long w4_trace[4][16][8][2];
 // the 2-byte output type; rows padded by 16 bytes when that does not fit a power-of-two swizzle).
 template <int BN, int MF>
 constexpr int w4_strip_pitch() { return BN == 256 ? 256 : BN + 16; }  // bytes per staged row (BN/2 columns of 2 bytes)
-template <int BN, int MF>
-constexpr int w4_lds_bytes() { return 2 * (256 + BN) * kRowBytes + 4 * 32 * w4_strip_pitch<BN, MF>(); }
+// AS = stages of the A operand's ring (B always has two).  With three, the epilogue strips hold 16 rows instead of 32
+// so that everything still fits the 160 KB of a CU.
+template <int BN, int MF, int AS = 2>
+constexpr int w4_lds_bytes() { return (AS * 256 + 2 * BN) * kRowBytes + 4 * (AS == 3 ? 16 : 32) * w4_strip_pitch<BN, MF>(); }
 
 // What the kernel needs from an epilogue besides bias_ptr(): finish(x) applied to acc + bias in fp32, and
 // dest8(m, n), the address of the 16 bytes that hold columns n..n+7 of output row m.
-template <typename T, int BN, int MF, typename Epi>
+//
+// AS = 3: the A operand (the activations: the matrix that comes from HBM or the memory-side cache, while the weights
+// stay in L2) gets a THIRD stage, so that its DMA loads are issued two K steps before the barrier that waits for them
+// instead of one.  With two stages a load has between half a K step and one K step (0.6-1.3 us) to land, which is
+// what an L2 hit takes and less than a fetch from HBM: the product whose A operand does not fit the memory-side
+// cache (the second FFN product: 201 MB) ran 20 % slower inside the forward than on a cache-resident operand.
+// The loads of a K step go out B first, A last; loads of one wavefront return in order, so the barrier waits for
+// all but the A_LOADS youngest (vmcnt(A_LOADS)): the weights of the next step and the activations of the next step
+// have landed, the activations of the step after it may still be in flight.  Global STORES return out of order with
+// loads, so the first barrier of a tile, which may still have the previous tile's stores in flight, waits for
+// everything.  Epilogues with a column pass keep two stages (their transposed unit needs the larger strip).
+template <typename T, int BN, int MF, typename Epi, int AS = 2>
 __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, const Epi epi) {
   static_assert(sizeof(T) == 2, "16-bit operands");
   static_assert(MF == 32 || MF == 16, "block sizes of the matrix instructions");
+  static_assert(AS == 2 || (AS == 3 && MF == 16 && !HasColumnPass<Epi>::value), "three A stages: 16-wide blocks, row-major epilogues");
   constexpr int BM = 256;
   constexpr int BK = kRowBytes / sizeof(T);
   constexpr int RB = 128 / MF, CB = BN / 2 / MF;   // blocks per wavefront: rows, columns
@@ -248,8 +283,9 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   const int lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm0 = (wave / 2) * 128, wn0 = (wave % 2) * (BN / 2);
   const int lrow = lane % MF, lgrp = lane / MF;
-  // LDS: [A stage 0][A stage 1][B stage 0][B stage 1][epilogue strips]; the stage of an operand is an immediate offset
-  const int a_row0 = (wm0 + lrow) * kRowBytes, b_row0 = 2 * A_BYTES + (wn0 + lrow) * kRowBytes;
+  // LDS: [A stage 0 .. AS-1][B stage 0][B stage 1][epilogue strips]; the stage of an operand is an immediate offset
+  // (with three A stages the A stage is a run-time offset)
+  const int a_row0 = (wm0 + lrow) * kRowBytes, b_row0 = AS * A_BYTES + (wn0 + lrow) * kRowBytes;
   const int swz = (lrow >> 1) & 7;
 
   // ---- DMA cursor.  `buffer_load_dwordx4 ... lds` copies 8 tile rows (64 lanes x 16 bytes) straight into LDS; the
@@ -293,7 +329,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       lds_char* as = lds0 + (dma_step & 1) * A_BYTES + wave * (A_LOADS * 1024);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, as + i * 1024, 16, voa[i], a_soff + dma_k * kRowBytes, 0, 0);
     } else {
-      lds_char* bs = lds0 + 2 * A_BYTES + (dma_step & 1) * B_BYTES + wave * (B_LOADS * 1024);
+      lds_char* bs = lds0 + AS * A_BYTES + (dma_step & 1) * B_BYTES + wave * (B_LOADS * 1024);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, bs + (i - A_LOADS) * 1024, 16, vob[i - A_LOADS], b_soff + dma_k * kRowBytes, 0, 0);
     }
   };
@@ -324,6 +360,66 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     }
   };
 
+  // ---- three A stages: one cursor per operand; the A cursor runs one K step ahead of the B cursor.  (voa / vob and
+  //      a_soff / b_soff above are then maintained by these, each at its own pace.)
+  int a_step = 0, a_k = 0, a_tile = first, a_st = 0;  // a_st = a_step % 3: the stage the cursor's step is loaded into
+  int b_step = 0, b_k = 0, b_tile = first;
+  auto a_point = [&](int tile) __attribute__((always_inline)) {
+    int tile_m, tile_n;
+    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM;
+    const int sub = lane >> 3, p = lane & 7;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int row = (wave * A_LOADS + i) * 8 + sub;
+      voa[i] = (uint32_t)(min(m0 + row, g.m - 1) - m0) * (uint32_t)lda_bytes + ((p ^ ((row >> 1) & 7)) << 4);
+    }
+    a_soff = (uint32_t)m0 * (uint32_t)lda_bytes;
+  };
+  auto b_point = [&](int tile) __attribute__((always_inline)) {
+    int tile_m, tile_n;
+    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int n0 = first_column(tile_n);
+    const int sub = lane >> 3, p = lane & 7;
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const int row = (wave * B_LOADS + i) * 8 + sub;
+      vob[i] = (uint32_t)(min(n0 + row, g.n - 1) - n0) * (uint32_t)ldb_bytes + ((p ^ ((row >> 1) & 7)) << 4);
+    }
+    b_soff = (uint32_t)n0 * (uint32_t)ldb_bytes;
+  };
+#if defined(__HIP_DEVICE_COMPILE__)
+  // load i of the split cursors: 0 .. B_LOADS-1 are the B loads (issued first), the rest the A loads
+  auto split_issue_one = [&](int i) __attribute__((always_inline)) {
+    if (i < B_LOADS) {
+      lds_char* bs = lds0 + AS * A_BYTES + (b_step & 1) * B_BYTES + wave * (B_LOADS * 1024);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, bs + i * 1024, 16, vob[i], b_soff + b_k * kRowBytes, 0, 0);
+    } else {
+      lds_char* as = lds0 + a_st * A_BYTES + wave * (A_LOADS * 1024);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, as + (i - B_LOADS) * 1024, 16, voa[i - B_LOADS], a_soff + a_k * kRowBytes, 0, 0);
+    }
+  };
+#else
+  auto split_issue_one = [&](int) {};
+#endif
+  auto a_advance = [&]() __attribute__((always_inline)) {
+    ++a_step;
+    a_st = a_st == 2 ? 0 : a_st + 1;
+    if (a_step < total_steps && ++a_k == ksteps) {
+      a_k = 0;
+      a_tile += stride;
+      a_point(a_tile);
+    }
+  };
+  auto b_advance = [&]() __attribute__((always_inline)) {
+    ++b_step;
+    if (b_step < total_steps && ++b_k == ksteps) {
+      b_k = 0;
+      b_tile += stride;
+      b_point(b_tile);
+    }
+  };
+
   Chunk fa[2][RB], fb[2][CB];
   auto read_frags = [&](int stage, int sub, Chunk (&a)[RB], Chunk (&b)[CB]) __attribute__((always_inline)) {
     const int off = ((sub * CPS + lgrp) ^ swz) << 4;
@@ -342,8 +438,9 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   // A scheduling fence after every MFMA keeps the compiler from regrouping them.
   // rd_stage/rd_sub: what the reads fetch; DLO: index of the first DMA load issued here.
   constexpr int READS = RB + CB, MMAS = RB * CB;
-  auto substep = [&](auto swap_tag, auto cur_tag, auto rd_stage_tag, auto rd_sub_tag, auto dlo_tag, auto nl_tag, auto ext_tag) __attribute__((always_inline)) {
+  auto substep = [&](auto swap_tag, auto cur_tag, auto rd_stage_tag, auto rd_sub_tag, auto dlo_tag, auto nl_tag, auto ext_tag, auto zero_tag) __attribute__((always_inline)) {
     constexpr bool SWAP = decltype(swap_tag)::value;
+    constexpr bool ZERO = decltype(zero_tag)::value;  // first substep of a tile: the accumulators are written, not added to
     constexpr int CUR = decltype(cur_tag)::value, RS = decltype(rd_stage_tag)::value, RSUB = decltype(rd_sub_tag)::value;
     constexpr int DLO = decltype(dlo_tag)::value, NL = decltype(nl_tag)::value, EXT = decltype(ext_tag)::value;  // NL loads over the first EXT MFMAs
     static_assert(NL <= EXT && EXT <= MMAS, "at most one DMA load per MFMA");
@@ -351,8 +448,13 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
 #pragma unroll
     for (int m = 0; m < MMAS; ++m) {
       const int i = m / CB, j = m % CB;
-      if constexpr (SWAP) MB::run(fb[CUR][j], fa[CUR][i], acc[i][j]);
-      else MB::run(fa[CUR][i], fb[CUR][j], acc[i][j]);
+      if constexpr (ZERO) {
+        if constexpr (SWAP) MB::run_zero(fb[CUR][j], fa[CUR][i], acc[i][j]);
+        else MB::run_zero(fa[CUR][i], fb[CUR][j], acc[i][j]);
+      } else {
+        if constexpr (SWAP) MB::run(fb[CUR][j], fa[CUR][i], acc[i][j]);
+        else MB::run(fa[CUR][i], fb[CUR][j], acc[i][j]);
+      }
       if (m < RB) fa[CUR ^ 1][m] = *reinterpret_cast<const Chunk*>(smem + (a_row0 + off) + (RS * A_BYTES + m * MF * kRowBytes));
       else if (m < READS) fb[CUR ^ 1][m - RB] = *reinterpret_cast<const Chunk*>(smem + (b_row0 + off) + (RS * B_BYTES + (m - RB) * MF * kRowBytes));
       if (NL > 0 && m < EXT && ((m + 1) * NL) / EXT != (m * NL) / EXT) dma_issue_one(DLO + (m * NL) / EXT);
@@ -370,25 +472,88 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   template_int<0> I0;
 
   // One K step.  P = parity of the step = its LDS stage.
-  auto k_step = [&](auto parity_tag, auto swap_tag) __attribute__((always_inline)) {
+  // zero_tag: the first K step of a tile (its first substep writes the accumulators instead of adding to them)
+  auto k_step = [&](auto parity_tag, auto swap_tag, auto zero_tag) __attribute__((always_inline)) {
     constexpr int P = decltype(parity_tag)::value;
+    std::false_type no;
     if constexpr (SUB == 4) {
-      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<1>{}, template_int<D3>{}, template_int<D0>{}, template_int<MMAS>{});
-      substep(swap_tag, template_int<1>{}, template_int<P>{}, template_int<2>{}, template_int<D3 + D0>{}, template_int<D1>{}, template_int<EXT1>{});
+      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<1>{}, template_int<D3>{}, template_int<D0>{}, template_int<MMAS>{}, zero_tag);
+      substep(swap_tag, template_int<1>{}, template_int<P>{}, template_int<2>{}, template_int<D3 + D0>{}, template_int<D1>{}, template_int<EXT1>{}, no);
       dma_advance();
       __builtin_amdgcn_sched_barrier(0);
-      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<3>{}, I0, I0, template_int<MMAS>{});
+      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<3>{}, I0, I0, template_int<MMAS>{}, no);
     } else {
-      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<1>{}, I0, I0, template_int<MMAS>{});
+      substep(swap_tag, template_int<0>{}, template_int<P>{}, template_int<1>{}, I0, I0, template_int<MMAS>{}, zero_tag);
       dma_advance();
       __builtin_amdgcn_sched_barrier(0);
     }
     // everyone has read all of this stage (the last reads were issued half a substep ago); the other stage has landed
     dma_landed_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    substep(swap_tag, template_int<1>{}, template_int<P ^ 1>{}, template_int<0>{}, I0, template_int<D3>{}, template_int<MMAS>{});
+    substep(swap_tag, template_int<1>{}, template_int<P ^ 1>{}, template_int<0>{}, I0, template_int<D3>{}, template_int<MMAS>{}, no);
   };
 
+  // ---- the same with three A stages (16-wide blocks, operands swapped).  a_rd: byte offset of the A stage that is
+  //      read.  ISSUE: the LOADS loads of the split cursors go out, evenly spread over the substep, B first.
+  auto substep3 = [&](auto cur_tag, auto rd_bstage_tag, auto rd_sub_tag, auto issue_tag, auto zero_tag, int a_rd) __attribute__((always_inline)) {
+    constexpr int CUR = decltype(cur_tag)::value, RSB = decltype(rd_bstage_tag)::value, RSUB = decltype(rd_sub_tag)::value;
+    constexpr bool ISSUE = decltype(issue_tag)::value, ZERO = decltype(zero_tag)::value;
+    const int off = ((RSUB * CPS + lgrp) ^ swz) << 4;
+    const int a_base = a_row0 + off + a_rd;
+#pragma unroll
+    for (int m = 0; m < MMAS; ++m) {
+      const int i = m / CB, j = m % CB;
+      if constexpr (ZERO) MB::run_zero(fb[CUR][j], fa[CUR][i], acc[i][j]);
+      else MB::run(fb[CUR][j], fa[CUR][i], acc[i][j]);
+      if (m < RB) fa[CUR ^ 1][m] = *reinterpret_cast<const Chunk*>(smem + a_base + m * MF * kRowBytes);
+      else if (m < READS) fb[CUR ^ 1][m - RB] = *reinterpret_cast<const Chunk*>(smem + (b_row0 + off) + (RSB * B_BYTES + (m - RB) * MF * kRowBytes));
+      if (ISSUE && ((m + 1) * LOADS) / MMAS != (m * LOADS) / MMAS) split_issue_one((m * LOADS) / MMAS);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  int a_cur = 0;  // stage (0..2) of the A operand of the K step being multiplied
+  auto k_step3 = [&](auto parity_tag, auto full_tag) __attribute__((always_inline)) {
+    constexpr int P = decltype(parity_tag)::value;
+    constexpr bool FULL = decltype(full_tag)::value;
+    // FULL = the first K step of a tile: its first substep also writes the accumulators instead of adding to them
+    substep3(template_int<0>{}, template_int<P>{}, template_int<1>{}, std::false_type{}, full_tag, a_cur * A_BYTES);
+    a_advance();
+    b_advance();
+    __builtin_amdgcn_sched_barrier(0);
+    // everyone has read all of this step's stages; the next step's operands have landed, the A loads of the step
+    // after it (the A_LOADS youngest of this wavefront) may still be in flight
+    if constexpr (FULL) dma_landed_barrier();
+    else dma_landed_barrier_but<A_LOADS>();
+    __builtin_amdgcn_sched_barrier(0);
+    a_cur = a_cur == 2 ? 0 : a_cur + 1;
+    substep3(template_int<1>{}, template_int<P ^ 1>{}, template_int<0>{}, std::true_type{}, std::false_type{}, a_cur * A_BYTES);
+  };
+  auto read_frags3 = [&](int a_rd) __attribute__((always_inline)) {  // sub 0 of (A stage at a_rd, B stage 0)
+    const int off = (lgrp ^ swz) << 4;
+#pragma unroll
+    for (int i = 0; i < RB; ++i) fa[0][i] = *reinterpret_cast<const Chunk*>(smem + (a_row0 + off + a_rd) + i * MF * kRowBytes);
+#pragma unroll
+    for (int j = 0; j < CB; ++j) fb[0][j] = *reinterpret_cast<const Chunk*>(smem + (b_row0 + off) + j * MF * kRowBytes);
+  };
+
+  if constexpr (AS == 3) {
+    // ---- prologue: A steps 0 and 1 and B step 0 land; B step 1 and A step 2 are under way ----
+    a_point(a_tile);
+    b_point(b_tile);
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) split_issue_one(B_LOADS + i);
+    a_advance();
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) split_issue_one(B_LOADS + i);
+    a_advance();
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) split_issue_one(i);
+    b_advance();
+    dma_landed_barrier();
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) split_issue_one(i);
+    read_frags3(0);
+  } else {
   // ---- prologue: K step 0 lands, the first loads of K step 1 are under way ----
   dma_point(dma_tile);
   dma_issue(std::integral_constant<int, 0>{}, std::integral_constant<int, LOADS>{});
@@ -396,8 +561,10 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   dma_landed_barrier();
   dma_issue(std::integral_constant<int, 0>{}, std::integral_constant<int, D3>{});
   read_frags(0, 0, fa[0], fb[0]);
+  }
 
-  char* strip = smem + 2 * STAGE + wave * (32 * PITCH);
+  constexpr int STRIP_ROWS = AS == 3 ? 16 : 32;
+  char* strip = smem + AS * A_BYTES + 2 * B_BYTES + wave * (STRIP_ROWS * PITCH);
   const uint32_t strip_lds = (uint32_t)reinterpret_cast<uintptr_t>(strip);  // low half of a generic LDS address = LDS offset
   int tile = first;
   for (int t = 0; t < my_tiles; ++t, tile += stride) {
@@ -408,13 +575,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     if constexpr (HasColumnPass<Epi>::value) swap = !(epi.column_pass() && n0 >= epi.first_column_of_pass());
     W4_STAMP(0)
 
-#pragma unroll
-    for (int i = 0; i < RB; ++i)
-#pragma unroll
-      for (int j = 0; j < CB; ++j)
-#pragma unroll
-        for (int e = 0; e < ACC; ++e) acc[i][j][e] = 0;
-
+    // (no zeroing of the accumulators: the first substep of the tile writes them)
     const auto* bias = epi.bias_ptr();
     using BiasT = typename std::remove_cv<typename std::remove_pointer<decltype(bias)>::type>::type;
     const int m_lim = g.m, n_lim = tile_n < g.split_tiles ? g.split_col : g.n;  // a tile in front of the split ends there
@@ -424,7 +585,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     // (16-row block v / (CB/2) of the group, pair of block columns v % (CB/2)), the lane's row is 16*(v / (CB/2)) + lrow.
     // (the widest tile of the 16-wide blocks stages 16 rows at a time: half the registers for the staged pieces, which
     // its head-split epilogue does not have to spare)
-    constexpr int GROUP = (MF == 16 && BN > 192) ? 16 : 32;
+    constexpr int GROUP = (AS == 3 || (MF == 16 && BN > 192)) ? 16 : 32;
     constexpr int NV = MF == 32 ? CB * 2 : (GROUP == 32 ? CB : CB / 2);
     constexpr int NBV = MF == 32 ? NV : CB / 2;  // distinct column groups among the units (= bias vectors to hold)
     auto unit_chunk = [&](int v) __attribute__((always_inline)) {  // which group of eight columns of the wavefront's BN/2
@@ -438,17 +599,25 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     }
     W4_STAMP(1)
     if (swap) {
-#ifdef TTMI_W4_TRACE
-      k_step(std::integral_constant<int, 0>{}, std::true_type{});
-      W4_STAMP(4)
-      k_step(std::integral_constant<int, 1>{}, std::true_type{});
-      W4_STAMP(5)
+      // the first two K steps apart: the very first substep writes the accumulators, and (three A stages) the first
+      // barrier of a tile, which may have the previous tile's stores in flight, waits for everything
+      if constexpr (AS == 3) {
+        k_step3(template_int<0>{}, std::true_type{});
+        k_step3(template_int<1>{}, std::false_type{});
+      } else {
+        k_step(std::integral_constant<int, 0>{}, std::true_type{}, std::true_type{});
+        W4_STAMP(4)
+        k_step(std::integral_constant<int, 1>{}, std::true_type{}, std::false_type{});
+        W4_STAMP(5)
+      }
       for (int kt = 2; kt < ksteps; kt += 2) {
-#else
-      for (int kt = 0; kt < ksteps; kt += 2) {
-#endif
-        k_step(std::integral_constant<int, 0>{}, std::true_type{});
-        k_step(std::integral_constant<int, 1>{}, std::true_type{});
+        if constexpr (AS == 3) {
+          k_step3(template_int<0>{}, std::false_type{});
+          k_step3(template_int<1>{}, std::false_type{});
+        } else {
+          k_step(std::integral_constant<int, 0>{}, std::true_type{}, std::false_type{});
+          k_step(std::integral_constant<int, 1>{}, std::true_type{}, std::false_type{});
+        }
       }
       W4_STAMP(2)
       // A lane now owns, per block, runs of four consecutive columns of one row; a pair swap makes them runs of
@@ -580,9 +749,11 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       }
     } else {
       if constexpr (HasColumnPass<Epi>::value) {
-        for (int kt = 0; kt < ksteps; kt += 2) {
-          k_step(std::integral_constant<int, 0>{}, std::false_type{});
-          k_step(std::integral_constant<int, 1>{}, std::false_type{});
+        k_step(std::integral_constant<int, 0>{}, std::false_type{}, std::true_type{});
+        k_step(std::integral_constant<int, 1>{}, std::false_type{}, std::false_type{});
+        for (int kt = 2; kt < ksteps; kt += 2) {
+          k_step(std::integral_constant<int, 0>{}, std::false_type{}, std::false_type{});
+          k_step(std::integral_constant<int, 1>{}, std::false_type{}, std::false_type{});
         }
         W4_STAMP(2)
         // A lane owns column lrow of every block and, after the pair swap, eight consecutive rows of it: one 16-byte
@@ -592,7 +763,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
         // eight adjacent lanes holding the 128 contiguous bytes of one column.  As in the row path, the arithmetic
         // of unit u runs while the strip reads of unit u-1 are in flight.
         constexpr int VT_PITCH = 144, UNITS = (BN / 2 / 32) * 2, VP = 4;  // unit = (32 columns, half of the 128 rows)
-        static_assert(32 * VT_PITCH <= 32 * PITCH, "the transposed unit fits the strip");
+        static_assert(32 * VT_PITCH <= STRIP_ROWS * PITCH, "the transposed unit fits the strip");
         float bj[CB];
         load_bias_columns_stride<CB, MF>(epi, n0 + wn0 + lrow, n_lim, bj);
         const int rd_col = lane >> 3, rd_chunk = lane & 7;  // pass p returns rows 8*rd_chunk.. of column 8*p + rd_col
@@ -683,7 +854,8 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     // here (K step 0 of the next tile sits untouched in stage 0 until that tile's own loads overwrite it) ends the
     // life of those registers at the end of the K loop, so the epilogue has them: up to 64 with 16-wide blocks.
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(0, 0, fa[0], fb[0]);
+    if constexpr (AS == 3) read_frags3(a_cur * A_BYTES);
+    else read_frags(0, 0, fa[0], fb[0]);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // surplus DMA loads have landed before the LDS is given back
 }
@@ -705,11 +877,18 @@ static bool w4_output_fits(const GemmArgs& g, int64_t ldc) {
 }
 
 // split_col: a column (multiple of 8) at which a fresh tile has to start whatever BN is (0 = none).
-template <typename T, int BN, typename Epi>
+// Three A stages where they fit (192-wide tiles, row-major epilogues).  Switch TTMI_W4_A_STAGES = 2 keeps two.
+template <int BN, typename Epi>
+constexpr bool w4_three_stages_fit() { return BN == 192 && !HasColumnPass<Epi>::value; }
+
+template <typename T, int BN, typename Epi, int AS = 2>
 static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s, int split_col = 0) {
-  constexpr int LDS = w4_lds_bytes<BN, kW4Block>();
+  if constexpr (AS == 2 && w4_three_stages_fit<BN, Epi>()) {
+    if (kernel_switch(kSwitchW4AStages) != 2) return launch_w4<T, BN, Epi, 3>(g, epi, s, split_col);
+  }
+  constexpr int LDS = w4_lds_bytes<BN, kW4Block, AS>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
-  if (describe_only("dma_agpr", 4, 256, BN)) return 0;
+  if (describe_only(AS == 3 ? "dma3_agpr" : "dma_agpr", 4, 256, BN)) return 0;
   g.tiles_m = (g.m + 255) / 256;
   g.split_col = split_col;
   g.split_tiles = split_col > 0 ? (split_col + BN - 1) / BN : 0;
@@ -718,7 +897,7 @@ static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s, int split_col = 
   TTMI_REQUIRE(tiles < (1ll << 30), "GEMM grid too large");
   // one persistent workgroup per CU (the LDS allows no second one), a multiple of the XCD count
   const unsigned grid = (unsigned)(std::min<int64_t>(ceil_div(tiles, kNumXcd), std::max(1, compute_units() / kNumXcd)) * kNumXcd);
-  auto kern = gemm_w4_kernel<T, BN, kW4Block, Epi>;
+  auto kern = gemm_w4_kernel<T, BN, kW4Block, Epi, AS>;
   const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
   if (rc != 0) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kW4Threads), LDS, s, g, epi);

@@ -575,7 +575,28 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     if constexpr (HasColumnPass<Epi>::value) swap = !(epi.column_pass() && n0 >= epi.first_column_of_pass());
     W4_STAMP(0)
 
-    // (no zeroing of the accumulators: the first substep of the tile writes them)
+    // Three A stages: no zeroing, the first substep of the tile writes the accumulators.  Two stages: zeroed here
+    // (peeling the first K step off the loop for a zero-addend form costs this variant twenty registers, which its
+    // 256-wide forms do not have).  The matrix instructions are inline asm, so the compiler does not know to keep the
+    // wait states between these register writes and the instruction that reads them as its addend: every accumulator
+    // is pinned as written (an empty asm that names it) before a pause that covers the distance.
+    if constexpr (AS != 3) {
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < CB; ++j)
+#pragma unroll
+          for (int e = 0; e < ACC; ++e) acc[i][j][e] = 0;
+      // (not in the head-split kernels: pinned, they spill 0.7-1.3 KB of registers per lane; their zeroing stays
+      // where the compiler puts it, which the bit-exact parity tests of those kernels watch)
+      if constexpr (!HasColumnPass<Epi>::value) {
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+          for (int j = 0; j < CB; ++j) asm volatile("" : "+a"(acc[i][j]));
+        asm volatile("s_nop 7");
+      }
+    }
     const auto* bias = epi.bias_ptr();
     using BiasT = typename std::remove_cv<typename std::remove_pointer<decltype(bias)>::type>::type;
     const int m_lim = g.m, n_lim = tile_n < g.split_tiles ? g.split_col : g.n;  // a tile in front of the split ends there
@@ -599,18 +620,13 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
     }
     W4_STAMP(1)
     if (swap) {
-      // the first two K steps apart: the very first substep writes the accumulators, and (three A stages) the first
+      // three A stages: the first two K steps apart; the very first substep writes the accumulators, and the first
       // barrier of a tile, which may have the previous tile's stores in flight, waits for everything
       if constexpr (AS == 3) {
         k_step3(template_int<0>{}, std::true_type{});
         k_step3(template_int<1>{}, std::false_type{});
-      } else {
-        k_step(std::integral_constant<int, 0>{}, std::true_type{}, std::true_type{});
-        W4_STAMP(4)
-        k_step(std::integral_constant<int, 1>{}, std::true_type{}, std::false_type{});
-        W4_STAMP(5)
       }
-      for (int kt = 2; kt < ksteps; kt += 2) {
+      for (int kt = AS == 3 ? 2 : 0; kt < ksteps; kt += 2) {
         if constexpr (AS == 3) {
           k_step3(template_int<0>{}, std::false_type{});
           k_step3(template_int<1>{}, std::false_type{});
@@ -749,9 +765,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       }
     } else {
       if constexpr (HasColumnPass<Epi>::value) {
-        k_step(std::integral_constant<int, 0>{}, std::false_type{}, std::true_type{});
-        k_step(std::integral_constant<int, 1>{}, std::false_type{}, std::false_type{});
-        for (int kt = 2; kt < ksteps; kt += 2) {
+        for (int kt = 0; kt < ksteps; kt += 2) {
           k_step(std::integral_constant<int, 0>{}, std::false_type{}, std::false_type{});
           k_step(std::integral_constant<int, 1>{}, std::false_type{}, std::false_type{});
         }

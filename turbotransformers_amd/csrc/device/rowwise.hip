@@ -80,12 +80,18 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
       Vec<T, VEC> g = load_vec<T, VEC>(gamma + col);
       Vec<T, VEC> b = load_vec<T, VEC>(beta + col);
       Vec<T, VEC> o;
+      float y[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        float y = to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean);
-        if (RES32) asm volatile("" : "+v"(y));  // out is the rounding of the fp32 value, not of the exact multiply-add
-        o.v[j] = from_float<T>(y);
-        if (RES32) out32[row * n + col + j] = y;
+        y[j] = to_float(b.v[j]) + to_float(g.v[j]) * rstd * (x[it][j] - mean);
+        if (RES32) asm volatile("" : "+v"(y[j]));  // out is the rounding of the fp32 value, not of the exact multiply-add
+      }
+      // (the stores in loops of their own: an asm statement between two stores keeps them from being merged)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(y[j]);
+      if (RES32) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out32[row * n + col + j] = y[j];
       }
       store_vec<T, VEC>(orow + col, o);
     }

@@ -354,7 +354,7 @@ TTMI_API int ttmi_gemm_fused(const void* a, const void* b, void* c, int64_t m, i
 
 /* Which kernel variant ttmi_gemm (epilogue TTMI_EPI_NONE, args NULL) or ttmi_gemm_fused would launch for an
  * aligned, densely packed product of this shape, as text: family (reg = register-staged, dma = global->LDS DMA,
- * dma_agpr = DMA with accumulators in AGPRs, wave = one wavefront per tile with its operand fragments straight from
+ * dma_agpr = DMA with accumulators in AGPRs, dma3_agpr = the same with a third LDS stage for the A operand, wave = one wavefront per tile with its operand fragments straight from
  * global memory), wavefronts per workgroup, tile, K split; e.g. "dma8w_256x256", "wave1w_32x32_splitk3".
  * Nothing is launched.  No counterpart in the reference (cuBLAS picks its kernels out of sight); measurement
  * scripts use it to tie recorded per-kernel figures to the variant they were recorded on.  For the QKV epilogues
@@ -388,6 +388,28 @@ TTMI_API int ttmi_yardstick_mfma(int block, int dtype, const void* operands, int
  *   activation, as ttmi_add_bias_act would after the bias (the FusedAddBiasGELU step of QBertIntermediate).  Together they stand in for the dynamically
  *   quantised Linear module the reference's QBert* layers call (qmodeling_bert.py:17,35). */
 #define TTMI_QUANT_SCALE_FLOATS 514
+/* Per-workgroup maxima handed from the kernel that PRODUCES an activation to the quantisation of the Linear that
+ * consumes it, so that finding the dynamic scale costs no pass (and no launch) of its own:
+ *   absmax_slots   DEVICE float[TTMI_ABSMAX_SLOTS]; a producer writes EVERY slot on every launch (max|output| of one
+ *                  workgroup each, zero in the rest): nothing has to be cleared and nothing carries over between calls;
+ *   slots_written  HOST int: TTMI_ABSMAX_SLOTS when the launch filled the slots, 0 when its workgroups outnumber
+ *                  them (then the slots are untouched and the consumer calls ttmi_quantize_rows_i8 as before).
+ * ttmi_add_bias_layer_norm_absmax   = ttmi_add_bias_layer_norm, the same bits in `out`;
+ * ttmi_gemm_i8_dequant_absmax       = ttmi_gemm_i8_dequant, the same bits in `c` (maximum taken after the activation);
+ * ttmi_quantize_rows_i8_from_absmax = the second half of ttmi_quantize_rows_i8: scale from the slots' maximum,
+ *                                     scale_dev[0] / [1] as there, the same bits in `q`.
+ * No counterpart in the reference, whose quantized Linear is its framework's dynamic quantisation
+ * (qmodeling_bert.py:17,35). */
+#define TTMI_ABSMAX_SLOTS 1024
+TTMI_API int ttmi_add_bias_layer_norm_absmax(void* out, const void* input, const void* bias, const void* gamma,
+                                             const void* beta, int64_t m, int64_t n, float eps, int dtype,
+                                             float* absmax_slots, int* slots_written, void* stream);
+TTMI_API int ttmi_gemm_i8_dequant_absmax(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev,
+                                         const float* w_scale, const float* bias, int act, int64_t m, int64_t n,
+                                         int64_t k, int64_t lda, int64_t ldb, int64_t ldc, float* absmax_slots,
+                                         int* slots_written, void* stream);
+TTMI_API int ttmi_quantize_rows_i8_from_absmax(const float* x, int8_t* q, float* scale_dev, const float* absmax_slots,
+                                               int64_t m, int64_t k, void* stream);
 /* ttmi_quantize_weight_rows_i8: per-output-channel symmetric scales for a weight w[N,K] (fp32):
  *   scales[n] = max_k |w[n,k]| / 127 (1 if the row is zero), q[n,k] = clamp(rint(w[n,k]/scales[n]), -127, 127). */
 TTMI_API int ttmi_quantize_weight_rows_i8(const float* w, int8_t* q, float* scales, int64_t n, int64_t k,

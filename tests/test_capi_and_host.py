@@ -236,7 +236,7 @@ def test_gemm_describe_names_the_variant_without_a_device():
     for m, n, k, epi in [(32768, 3072, 768, capi.EPI_BIAS_ACT), (32768, 768, 3072, capi.EPI_NONE), (128, 768, 3072, capi.EPI_NONE),
                          (2560, 768, 3072, capi.EPI_BIAS)]:
         capi.check(lib.ttmi_gemm_describe(m, n, k, epi, ctypes.byref(args), capi.F16, buf, 64))
-        assert re.fullmatch(r"(reg|dma|dma_agpr|wave)\d+w_\d+x\d+(_splitk\d+)?", buf.value.decode()), buf.value
+        assert re.fullmatch(r"(reg|dma|dma_agpr|dma3_agpr|wave)\d+w_\d+x\d+(_splitk\d+)?", buf.value.decode()), buf.value
     assert lib.ttmi_gemm_describe(128, 768, 3072, capi.EPI_NONE, None, capi.F16, buf, 4) != 0  # too small for the answer
 
 

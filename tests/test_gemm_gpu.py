@@ -566,6 +566,40 @@ def test_gemm_i8_dequant_qkv_split_equals_the_two_kernels(ttmi, oracle, B, S, h,
         assert max_abs(host(x), y) <= 1e-5 * max(1.0, float(np.abs(y).max()))
 
 
+@pytest.mark.parametrize("M,N,K,act", [(2560, 3072, 768, capi.ACT_GELU), (2560, 768, 3072, -1), (200, 384, 256, capi.ACT_GELU),
+                                       (777, 100, 64, -1), (40000, 64, 64, -1)])
+def test_gemm_i8_dequant_leaves_the_maxima_for_the_next_quantisation(ttmi, M, N, K, act):
+    """ttmi_gemm_i8_dequant_absmax: the bits of ttmi_gemm_i8_dequant in c, and, when the launch filled the slots, every
+    slot written (they start as NaN here: nothing needs clearing), their maximum exactly max|c|; quantising c from the
+    slots gives the bits and the scale of the two-launch quantisation.  A launch with more workgroups than slots
+    says so and leaves the slots alone (see the LayerNorm form of this test for a case that does)."""
+    import ctypes
+    rng = np.random.default_rng(M + N)
+    a = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    b = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    sx, sw = np.array([0.0123, 0.0], np.float32), (rng.random(N, np.float32) + 0.5) * 1e-3
+    bias = rng.standard_normal(N).astype(np.float32)
+    dA, dB, dsx, dsw, dbias = dev(a), dev(b), dev(sx), dev(sw), dev(bias)
+    plain, fused = torch.empty((M, N), device="cuda"), torch.empty((M, N), device="cuda")
+    slots = torch.full((capi.ABSMAX_SLOTS, ), float("nan"), device="cuda")
+    written = ctypes.c_int(-1)
+    ok(ttmi.ttmi_gemm_i8_dequant(ptr(dA), ptr(dB), ptr(plain), ptr(dsx), ptr(dsw), ptr(dbias), act, M, N, K, K, K, N, stream()))
+    ok(ttmi.ttmi_gemm_i8_dequant_absmax(ptr(dA), ptr(dB), ptr(fused), ptr(dsx), ptr(dsw), ptr(dbias), act, M, N, K, K, K, N,
+                                        ptr(slots), ctypes.byref(written), stream()))
+    assert torch.equal(fused, plain)
+    if written.value == 0:  # (whether a shape's launch fits the slots is the tile picker's business)
+        assert torch.isnan(slots).all()
+        return
+    assert written.value == capi.ABSMAX_SLOTS
+    assert not torch.isnan(slots).any() and float(slots.min()) >= 0.0
+    assert float(slots.max()) == float(plain.abs().max())
+    q1, q2 = (torch.empty((M, N), dtype=torch.int8, device="cuda") for _ in range(2))
+    s1, s2 = (torch.full((capi.QUANT_SCALE_FLOATS, ), float("nan"), device="cuda") for _ in range(2))
+    ok(ttmi.ttmi_quantize_rows_i8(ptr(plain), ptr(q1), ptr(s1), M, N, stream()))
+    ok(ttmi.ttmi_quantize_rows_i8_from_absmax(ptr(plain), ptr(q2), ptr(s2), ptr(slots), M, N, stream()))
+    assert torch.equal(q1, q2) and torch.equal(s1[:2], s2[:2])
+
+
 def test_int8_linear_pipeline(ttmi, oracle):
     """quantize -> int8 GEMM -> dequant+bias, against the oracle's statement of the same scheme."""
     rng = np.random.default_rng(3)

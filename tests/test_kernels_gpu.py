@@ -74,6 +74,32 @@ def test_add_bias_layer_norm_fp32_product(ttmi, oracle, dt, m, n):
                                                    stream()) == -1
 
 
+@pytest.mark.parametrize("dt", ALL_DTYPES)
+@pytest.mark.parametrize("m,n", [(2560, 768), (37, 768), (3, 1024), (9000, 768), (5, 770)])
+def test_add_bias_layer_norm_leaves_the_maxima_for_the_next_quantisation(ttmi, dt, m, n):
+    """ttmi_add_bias_layer_norm_absmax: the bits of ttmi_add_bias_layer_norm in out, and the slots' maximum is
+    max|out|; with more workgroups than slots, or on the one-workgroup-per-row fallback, it reports 0 slots and
+    leaves them alone."""
+    import ctypes
+    from turbotransformers_amd import capi
+    rng = np.random.default_rng(m + n)
+    out, inp = rng.standard_normal((m, n), np.float32), rng.standard_normal((m, n), np.float32)
+    vecs = [dev(rng.standard_normal(n).astype(np.float32), dt) for _ in range(3)]
+    a, b, d_in = dev(out, dt), dev(out, dt), dev(inp, dt)
+    ok(ttmi.ttmi_add_bias_layer_norm(ptr(a), ptr(d_in), *[ptr(v) for v in vecs], m, n, 1e-12, TTMI_DTYPES[dt], stream()))
+    slots = torch.full((capi.ABSMAX_SLOTS, ), float("nan"), device="cuda")
+    written = ctypes.c_int(-1)
+    ok(ttmi.ttmi_add_bias_layer_norm_absmax(ptr(b), ptr(d_in), *[ptr(v) for v in vecs], m, n, 1e-12, TTMI_DTYPES[dt], ptr(slots),
+                                            ctypes.byref(written), stream()))
+    assert torch.equal(a, b)
+    if written.value == 0:
+        assert (m, n) in ((9000, 768), (5, 770)) and torch.isnan(slots).all()
+    else:
+        assert written.value == capi.ABSMAX_SLOTS
+        assert not torch.isnan(slots).any()
+        assert float(slots.max()) == float(a.float().abs().max())
+
+
 @pytest.mark.parametrize("n", [768, 1000, 4096])
 def test_layer_norm_of_near_constant_rows_stays_finite(ttmi, n):
     """E[x^2] - mean^2 (the reference's formula, layer_norm.cpp:144-163) cancels on a row whose spread is far below its

@@ -21,6 +21,7 @@ ACT_GELU, ACT_TANH, ACT_RELU = range(3)
 H2D, D2H, D2D = range(3)
 EPI_NONE, EPI_BIAS, EPI_BIAS_ACT, EPI_BIAS_RESIDUAL, EPI_QKV_SPLIT, EPI_QKV_SPLIT_PAD, EPI_F32_OUT = range(7)
 QUANT_SCALE_FLOATS = 514  # TTMI_QUANT_SCALE_FLOATS
+ABSMAX_SLOTS = 1024  # TTMI_ABSMAX_SLOTS
 
 
 class EpilogueArgs(ctypes.Structure):

@@ -278,9 +278,9 @@ int ttmi_gemm_i8(const int8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_
   return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
 }
 
-int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev, const float* w_scale,
-                         const float* bias, int act, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc,
-                         void* stream) {
+static int gemm_i8_dequant_impl(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev, const float* w_scale,
+                                const float* bias, int act, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                                int64_t ldc, float* absmax_slots, void* stream) {
   TTMI_REQUIRE(a && b && c && act_scale_dev && w_scale, "null tensor");
   TTMI_REQUIRE(act >= TTMI_ACT_NONE && act <= TTMI_ACT_RELU, "unknown activation");
   TTMI_REQUIRE(m < (1ll << 31) && n < (1ll << 31) && k < (1ll << 31), "dimension too large");
@@ -291,9 +291,28 @@ int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float
   g.m = (int)m; g.n = (int)n; g.k = (int)k;
   g.lda = lda; g.ldb = ldb;
   g.inner = 1;
-  EpiDequant epi{c, act_scale_dev, w_scale, bias, ldc, aligned16(c) && ldc % 4 == 0, act};
+  EpiDequant epi{c, act_scale_dev, w_scale, bias, ldc, aligned16(c) && ldc % 4 == 0, act, absmax_slots};
   const bool aligned = aligned16(a) && aligned16(b) && lda % 16 == 0 && ldb % 16 == 0 && k % 16 == 0;
   return launch_gemm<int8_t, false>(g, epi, 1, aligned, (hipStream_t)stream);
+}
+
+int ttmi_gemm_i8_dequant(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev, const float* w_scale,
+                         const float* bias, int act, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb, int64_t ldc,
+                         void* stream) {
+  return gemm_i8_dequant_impl(a, b, c, act_scale_dev, w_scale, bias, act, m, n, k, lda, ldb, ldc, nullptr, stream);
+}
+
+int ttmi_gemm_i8_dequant_absmax(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev, const float* w_scale,
+                                const float* bias, int act, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                                int64_t ldc, float* absmax_slots, int* slots_written, void* stream) {
+  TTMI_REQUIRE(absmax_slots && slots_written, "null absmax arguments");
+  static_assert(kAbsmaxSlots == TTMI_ABSMAX_SLOTS, "slot count of the C ABI");
+  tl_absmax_written = 0;
+  *slots_written = 0;
+  if (m <= 0 || n <= 0) return 0;
+  const int rc = gemm_i8_dequant_impl(a, b, c, act_scale_dev, w_scale, bias, act, m, n, k, lda, ldb, ldc, absmax_slots, stream);
+  *slots_written = rc == 0 ? tl_absmax_written : 0;
+  return rc;
 }
 
 int ttmi_gemm_i8_dequant_qkv_split(const int8_t* a, const int8_t* b, const float* act_scale_dev, const float* w_scale,

@@ -439,23 +439,23 @@ struct EpiDequant {
   int64_t ldc;
   bool vec;
   int act;  // ttmi_act, applied after the bias
+  // Optional: kAbsmaxSlots floats that receive max|output| per workgroup (slot = workgroup id, the rest zero), so that
+  // the dynamic quantisation of the NEXT Linear's input needs no pass of its own to find its scale.
+  float* absmax;
   __device__ __forceinline__ const float* bias_ptr() const { return bias; }
   __device__ __forceinline__ bool has_bias() const { return bias != nullptr; }
-  // v: the bit patterns of the dequantised values (dequantise() below, applied in accumulator layout)
+  __host__ __device__ __forceinline__ float* absmax_slots() const { return absmax; }
+  __device__ __forceinline__ float activate(float x) const {
+    if (act == TTMI_ACT_GELU) return apply_act<TTMI_ACT_GELU>(x);
+    if (act == TTMI_ACT_TANH) return apply_act<TTMI_ACT_TANH>(x);
+    if (act == TTMI_ACT_RELU) return apply_act<TTMI_ACT_RELU>(x);
+    return x;
+  }
+  // v: the bit patterns of the finished values (dequantise() and activate(), applied in accumulator layout)
   __device__ __forceinline__ void store8(int, int m, int n, int (&v)[8], int valid) const {
     float r[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) r[j] = __builtin_bit_cast(float, v[j]);
-    if (act == TTMI_ACT_GELU) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) r[j] = apply_act<TTMI_ACT_GELU>(r[j]);
-    } else if (act == TTMI_ACT_TANH) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) r[j] = apply_act<TTMI_ACT_TANH>(r[j]);
-    } else if (act == TTMI_ACT_RELU) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) r[j] = apply_act<TTMI_ACT_RELU>(r[j]);
-    }
     float* p = c + (int64_t)m * ldc + n;
     if (vec && valid == 8) {
       store_row8<float>(p, r);
@@ -475,6 +475,8 @@ struct EpiDequantQkvSplit {
   const float* w_scale;             // [N]
   __device__ __forceinline__ const float* bias_ptr() const { return split.bias; }
   __device__ __forceinline__ bool has_bias() const { return true; }
+  __host__ __device__ __forceinline__ float* absmax_slots() const { return nullptr; }
+  __device__ __forceinline__ float activate(float x) const { return x; }
   __device__ __forceinline__ void store8(int z, int m, int n, int (&v)[8], int valid) const {
     float r[8];
 #pragma unroll
@@ -499,6 +501,29 @@ __device__ __forceinline__ float dequantise(int acc, float act_scale, float w_sc
   float r = (float)acc * act_scale * w_scale;
   if (has_bias) r = r + bias;
   return r;
+}
+// Slots of the per-workgroup maxima a dequantising GEMM may leave for the quantisation of its consumer.
+constexpr int kAbsmaxSlots = 1024;
+// End of a workgroup's work: its maximum to its slot; workgroup 0 zeroes the slots no workgroup owns.  `red`: LDS the
+// kernel no longer needs (at least 16 floats).  Nothing has to be cleared beforehand and nothing is accumulated
+// across launches: every slot is written by every launch.
+template <typename Epi>
+__device__ __forceinline__ void publish_absmax(const Epi& epi, float lane_max, float* red, int threads) {
+  if constexpr (Dequantises<Epi>::value) {
+    float* slots = epi.absmax_slots();
+    if (slots == nullptr) return;
+    __syncthreads();
+    lane_max = group_max<kWave>(lane_max);
+    if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = lane_max;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float m = 0.f;
+      for (int w = 0; w < threads / kWave; ++w) m = fmaxf(m, red[w]);
+      slots[blockIdx.x] = m;
+    }
+    if (blockIdx.x == 0)
+      for (int i = (int)gridDim.x + (int)threadIdx.x; i < kAbsmaxSlots; i += threads) slots[i] = 0.f;
+  }
 }
 // sj[0..TN) = weight scales of the lane's columns, sj[TN] = activation scale; untouched for other epilogues
 template <int TN, typename Epi>
@@ -535,7 +560,7 @@ struct HasColumnPass<EpiQkvSplit<T, PAD>> : std::true_type {};
 template <typename T, int TM, int TN, int NT, int LDS_BYTES, typename Epi>
 __device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], const float (&bj)[TN], const float (&sj)[TN + 1],
                                            char* smem, const Epi& epi, const GemmArgs& g, int z, int wave_m0, int wave_n0,
-                                           int lane, int wave) {
+                                           int lane, int wave, float& amax) {
   using AccScalar = typename Mma<T>::AccScalar;
   constexpr int W = TN * 32;             // strip width (columns)
   constexpr int LDW = W + 4;             // padded pitch in words: rows stay 16-byte aligned
@@ -551,9 +576,11 @@ __device__ __forceinline__ void store_tile(typename Mma<T>::Acc (&acc)[TM][TN], 
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         AccScalar staged;
-        if constexpr (Dequantises<Epi>::value)
-          staged = __builtin_bit_cast(AccScalar, dequantise(acc[i][j][e], sj[TN], sj[j], bj[j], epi.has_bias()));
-        else
+        if constexpr (Dequantises<Epi>::value) {
+          const float r = epi.activate(dequantise(acc[i][j][e], sj[TN], sj[j], bj[j], epi.has_bias()));
+          amax = fmaxf(amax, fabsf(r));  // rows past M and columns past N repeat valid rows / are zero: harmless
+          staged = __builtin_bit_cast(AccScalar, r);
+        } else
           staged = acc[i][j][e] + (AccScalar)bj[j];
         stage[(8 * (e / 4) + 4 * lhalf + (e % 4)) * LDW + j * 32 + lrow] = staged;
       }
@@ -626,7 +653,11 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
   const bool remap = tiles >= kXcdRemapMinTiles;
   const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
   const int logical = remap ? (int)(blockIdx.x % kNumXcd) * per_xcd + (int)(blockIdx.x / kNumXcd) : (int)blockIdx.x;
-  if (logical >= tiles) return;
+  if (logical >= tiles) {
+    if constexpr (Dequantises<Epi>::value)
+      if (epi.absmax_slots() != nullptr && threadIdx.x == 0) epi.absmax_slots()[blockIdx.x] = 0.f;  // an idle workgroup still owns a slot
+    return;
+  }
   int tile_m, tile_n;
   tile_coords(logical, g.tiles_m, g.tiles_n, tile_m, tile_n);
   const int z = blockIdx.z;
@@ -780,7 +811,9 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_kernel(const GemmArgs g,
   float bj[TN], sj[TN + 1];
   load_bias_columns<TN>(epi, n0 + wn0 + lrow, g.n, bj);
   load_dequant_columns<TN>(epi, n0 + wn0 + lrow, g.n, sj);
-  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, bj, sj, smem, epi, g, z_epi, m0 + wm0, n0 + wn0, lane, wave);
+  float amax = 0.f;
+  store_tile<T, TM, TN, NT, 2 * STAGE>(acc, bj, sj, smem, epi, g, z_epi, m0 + wm0, n0 + wn0, lane, wave, amax);
+  publish_absmax(epi, amax, reinterpret_cast<float*>(smem), NT);
 }
 
 // ------------------------------------------------------------------ wavefront kernel -----
@@ -849,7 +882,8 @@ __global__ __launch_bounds__(kWave) void gemm_wave_kernel(const GemmArgs g, cons
       }
     }
   }
-  store_tile<T, 1, 1, kWave, STRIP>(acc, bj, sj, strip, epi, g, z_epi, m0, n0, lane, 0);
+  float amax = 0.f;  // (no dequantising epilogue takes this kernel)
+  store_tile<T, 1, 1, kWave, STRIP>(acc, bj, sj, strip, epi, g, z_epi, m0, n0, lane, 0, amax);
 }
 
 // ---------------------------------------------------------------------------- split-K -----
@@ -1071,7 +1105,11 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
   const int xcd = (int)(blockIdx.x % kNumXcd), stride = remap ? (int)(gridDim.x / kNumXcd) : (int)gridDim.x;
   const int xcd_end = remap ? min((xcd + 1) * per_xcd, tiles) : tiles;
   int logical = remap ? xcd * per_xcd + (int)(blockIdx.x / kNumXcd) : (int)blockIdx.x;
-  if (logical >= xcd_end) return;
+  if (logical >= xcd_end) {
+    if constexpr (Dequantises<Epi>::value)
+      if (epi.absmax_slots() != nullptr && threadIdx.x == 0) epi.absmax_slots()[blockIdx.x] = 0.f;  // an idle workgroup still owns a slot
+    return;
+  }
   const int z = blockIdx.z;
   const T* A = reinterpret_cast<const T*>(g.a) + (int64_t)(z / g.inner) * g.a_outer + (int64_t)(z % g.inner) * g.a_inner;
   const T* B = reinterpret_cast<const T*>(g.b) + (int64_t)(z / g.inner) * g.b_outer + (int64_t)(z % g.inner) * g.b_inner;
@@ -1175,6 +1213,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
 
   point_at(logical);
   issue(0);
+  float amax = 0.f;  // max |output| of this workgroup's tiles (dequantising epilogues)
   for (;;) {
     int tile_m, tile_n;
     tile_coords(logical, g.tiles_m, g.tiles_n, tile_m, tile_n);
@@ -1238,10 +1277,11 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_fast_kernel(const GemmAr
       __builtin_amdgcn_s_waitcnt(0x0F70);
     }
     store_tile<T, TM, TN, NT, fast_lds_bytes<BM, BN, WM, WN, NS>() - STAGE>(acc, bj, sj, smem + STAGE, epi, g, z_epi, m0 + wm0,
-                                                                             n0 + wn0, lane, wave);
+                                                                             n0 + wn0, lane, wave, amax);
     if (next >= xcd_end) break;
     logical = next;
   }
+  publish_absmax(epi, amax, reinterpret_cast<float*>(smem), NT);
 }
 
 // ------------------------------------------------------------------------ launching -----
@@ -1254,6 +1294,25 @@ static bool describe_only(const char* family, int waves, int bm, int bn, int spl
   *tl_describe = std::string(family) + std::to_string(waves) + "w_" + std::to_string(bm) + "x" + std::to_string(bn);
   if (splits > 1) *tl_describe += "_splitk" + std::to_string(splits);
   return true;
+}
+
+// A dequantising epilogue that was asked for per-workgroup maxima gets them only from a launch whose workgroups fit
+// the slots; otherwise the request is dropped and the caller told (tl_absmax_written stays 0), and it finds the
+// maximum with a pass of its own.
+static thread_local int tl_absmax_written = 0;
+template <typename Epi>
+static bool absmax_grid_ok(const Epi& epi, unsigned grid_x, int batch) {
+  if constexpr (Dequantises<Epi>::value) {
+    if (epi.absmax_slots() == nullptr) return true;
+    if (grid_x > (unsigned)kAbsmaxSlots || batch != 1) return false;
+    tl_absmax_written = kAbsmaxSlots;
+  }
+  return true;
+}
+template <typename Epi>
+static Epi without_absmax(Epi epi) {
+  if constexpr (std::is_same<Epi, EpiDequant>::value) epi.absmax = nullptr;
+  return epi;
 }
 
 // Kernels that use more than 64 KB of dynamic LDS need the limit raised once per kernel and device.
@@ -1280,6 +1339,7 @@ static int launch_config(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
   TTMI_REQUIRE(tiles < (1ll << 30) && batch < 65536, "GEMM grid too large");
   const unsigned grid_x = tiles >= kXcdRemapMinTiles ? (unsigned)(ceil_div(tiles, kNumXcd) * kNumXcd) : (unsigned)tiles;
   constexpr int DEPTH = (BM * BN <= 64 * 64 && ALIGNED) ? 2 : 1;
+  if (!absmax_grid_ok(epi, grid_x, batch)) return launch_config<T, BM, BN, WM, WN, B_KN, ALIGNED>(g, without_absmax(epi), batch, s);
   auto kern = gemm_kernel<T, BM, BN, WM, WN, B_KN, ALIGNED, DEPTH, Epi>;
   if (LDS > 64 * 1024) {
     const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
@@ -1317,6 +1377,7 @@ static int launch_fast(GemmArgs g, const Epi& epi, int batch, hipStream_t s) {
       tiles >= kXcdRemapMinTiles
           ? (unsigned)(std::min(ceil_div(tiles, kNumXcd), std::max<int64_t>(1, resident / kNumXcd)) * kNumXcd)
           : (unsigned)tiles;
+  if (!absmax_grid_ok(epi, grid_x, batch)) return launch_fast<T, BM, BN, WM, WN, Epi, NS>(g, without_absmax(epi), batch, s);
   auto kern = gemm_fast_kernel<T, BM, BN, WM, WN, NS, Epi>;
   if (LDS > 64 * 1024) {
     const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);

@@ -40,10 +40,12 @@ __device__ __forceinline__ int quantize_one(float x, float scale) {
   return (int)r;
 }
 
+// partial: `partials` per-workgroup maxima of |x|, written by absmax_kernel (then scale_dev + 2) or by the kernel
+// that produced x.
 __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, int8_t* __restrict__ q,
-                                                       float* __restrict__ scale_dev, int partials, int64_t n) {
+                                                       float* __restrict__ scale_dev, const float* __restrict__ partial,
+                                                       int partials, int64_t n) {
   __shared__ float red[4];
-  const float* partial = scale_dev + 2;
   float mx = 0.f;
   for (int p = threadIdx.x; p < partials; p += 256) mx = fmaxf(mx, partial[p]);
   mx = block_max_256(mx, red);
@@ -132,8 +134,19 @@ int ttmi_quantize_rows_i8(const float* x, int8_t* q, float* scale_dev, int64_t m
   static_assert(kMaxPartials + 2 == TTMI_QUANT_SCALE_FLOATS, "scale_dev holds the scale, the maximum and the partial maxima");
   hipLaunchKernelGGL(absmax_kernel, dim3((unsigned)partials), dim3(256), 0, s, x, n, scale_dev + 2);
   const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(n, 256 * 4), 256 * 8);
-  hipLaunchKernelGGL(quantize_kernel, dim3(std::max(grid, 1u)), dim3(256), 0, s, x, q, scale_dev, partials, n);
+  hipLaunchKernelGGL(quantize_kernel, dim3(std::max(grid, 1u)), dim3(256), 0, s, x, q, scale_dev, scale_dev + 2, partials, n);
   return launch_status("quantize_rows_i8");
+}
+
+int ttmi_quantize_rows_i8_from_absmax(const float* x, int8_t* q, float* scale_dev, const float* absmax_slots, int64_t m,
+                                      int64_t k, void* stream) {
+  TTMI_REQUIRE(x && q && scale_dev && absmax_slots, "null tensor");
+  const int64_t n = m * k;
+  if (n <= 0) return 0;
+  const unsigned grid = (unsigned)std::min<int64_t>(ceil_div(n, 256 * 4), 256 * 8);
+  hipLaunchKernelGGL(quantize_kernel, dim3(std::max(grid, 1u)), dim3(256), 0, (hipStream_t)stream, x, q, scale_dev, absmax_slots,
+                     TTMI_ABSMAX_SLOTS, n);
+  return launch_status("quantize_rows_i8_from_absmax");
 }
 
 int ttmi_quantize_weight_rows_i8(const float* w, int8_t* q, float* scales, int64_t n, int64_t k, void* stream) {

@@ -20,12 +20,15 @@ constexpr int kBlock = 256;
 // encoder in fp32 -- only GEMM operands are rounded -- at the cost of 12 instead of 6 bytes/element.
 // RES32 = 2: in addition the product itself arrives unrounded, in `out32` (which this kernel then overwrites with
 // the result, element by element, each by the thread that read it); `out` is only written: 14 bytes/element.
+// absmax (optional): TTMI_ABSMAX_SLOTS floats; workgroup b writes max|result| of its rows to slot b and workgroup 0
+// zeroes the slots past the grid (the launcher passes it only when the grid fits), so that the dynamic quantisation
+// of the next Linear's input finds its scale without a pass of its own.
 template <typename T, int VEC, int G, int ITERS, bool ADD, int RES32>
 __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, const T* __restrict__ input,
                                                           const T* __restrict__ bias,
                                                           const T* __restrict__ gamma,
                                                           const T* __restrict__ beta, int64_t m, int n,
-                                                          float eps, const float* res32, float* out32) {
+                                                          float eps, const float* res32, float* out32, float* absmax) {
   constexpr int ROWS = kBlock / G;
   const int lane = threadIdx.x % G;
   const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / G;
@@ -73,6 +76,7 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
   const float mean = sum / (float)n;
   const float var = fmaxf(sumsq / (float)n - mean * mean, 0.f);  // cancellation on a near-constant row must not go negative
   const float rstd = 1.0f / sqrtf(var + eps);
+  float amax = 0.f;
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int col = (it * G + lane) * VEC;
@@ -88,13 +92,30 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows(T* __restrict__ out, c
       }
       // (the stores in loops of their own: an asm statement between two stores keeps them from being merged)
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) o.v[j] = from_float<T>(y[j]);
+      for (int j = 0; j < VEC; ++j) {
+        o.v[j] = from_float<T>(y[j]);
+        amax = fmaxf(amax, fabsf(to_float(o.v[j])));  // of the value as stored
+      }
       if (RES32) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) out32[row * n + col + j] = y[j];
       }
       store_vec<T, VEC>(orow + col, o);
     }
+  }
+  if (absmax != nullptr) {
+    __shared__ float red[kBlock / kWave];
+    amax = group_max<kWave>(amax);
+    if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float mx = 0.f;
+#pragma unroll
+      for (int w = 0; w < kBlock / kWave; ++w) mx = fmaxf(mx, red[w]);
+      absmax[blockIdx.x] = mx;
+    }
+    if (blockIdx.x == 0)
+      for (int i = (int)gridDim.x + (int)threadIdx.x; i < TTMI_ABSMAX_SLOTS; i += kBlock) absmax[i] = 0.f;
   }
 }
 
@@ -148,18 +169,21 @@ __global__ __launch_bounds__(kBlock) void layer_norm_block(T* __restrict__ out, 
 
 template <typename T, int VEC, int G, int ITERS, bool ADD, int RES32>
 static int launch_ln_rows(T* out, const T* input, const T* bias, const T* gamma, const T* beta, int64_t m,
-                          int n, float eps, const float* res32, float* out32, hipStream_t s) {
+                          int n, float eps, const float* res32, float* out32, hipStream_t s, float* absmax, int* slots_written) {
   constexpr int ROWS = kBlock / G;
   const int64_t grid = ceil_div(m, ROWS);
+  if (grid > TTMI_ABSMAX_SLOTS) absmax = nullptr;  // more workgroups than slots: the caller finds the maximum itself
+  if (slots_written != nullptr) *slots_written = absmax != nullptr ? TTMI_ABSMAX_SLOTS : 0;
   hipLaunchKernelGGL((layer_norm_rows<T, VEC, G, ITERS, ADD, RES32>), dim3((unsigned)grid), dim3(kBlock), 0, s,
-                     out, input, bias, gamma, beta, m, n, eps, res32, out32);
+                     out, input, bias, gamma, beta, m, n, eps, res32, out32, absmax);
   return launch_status("layer_norm_rows");
 }
 
 template <typename T, bool ADD, int RES32 = 0>
 static int layer_norm_dispatch(T* out, const T* input, const T* bias, const T* gamma, const T* beta,
                                int64_t m, int64_t n, float eps, hipStream_t s, const float* res32 = nullptr,
-                               float* out32 = nullptr) {
+                               float* out32 = nullptr, float* absmax = nullptr, int* slots_written = nullptr) {
+  if (slots_written != nullptr) *slots_written = 0;
   if (m == 0 || n == 0) return 0;
   constexpr int VEC = 16 / sizeof(T);
   auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
@@ -169,7 +193,7 @@ static int layer_norm_dispatch(T* out, const T* input, const T* bias, const T* g
     const int64_t nv = n / VEC;  // 16-byte vectors per row
     // Pick the group width G so that nv = G * ITERS with as little idle lane time as possible.
 #define TTMI_LN_CASE(G, ITERS) \
-  return launch_ln_rows<T, VEC, G, ITERS, ADD, RES32>(out, input, bias, gamma, beta, m, (int)n, eps, res32, out32, s)
+  return launch_ln_rows<T, VEC, G, ITERS, ADD, RES32>(out, input, bias, gamma, beta, m, (int)n, eps, res32, out32, s, absmax, slots_written)
     if (nv <= 16) TTMI_LN_CASE(16, 1);
     if (nv <= 32) TTMI_LN_CASE(32, 1);
     if (nv <= 64) TTMI_LN_CASE(64, 1);
@@ -411,6 +435,18 @@ int ttmi_add_bias_layer_norm(void* out, const void* input, const void* bias, con
   TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, true>((T*)out, (const T*)input, (const T*)bias,
                                                                       (const T*)gamma, (const T*)beta, m, n, eps,
                                                                       (hipStream_t)stream)));
+  return 0;
+}
+
+int ttmi_add_bias_layer_norm_absmax(void* out, const void* input, const void* bias, const void* gamma, const void* beta,
+                                    int64_t m, int64_t n, float eps, int dtype, float* absmax_slots, int* slots_written,
+                                    void* stream) {
+  TTMI_REQUIRE(out && input && bias && gamma && beta && absmax_slots && slots_written, "null tensor");
+  TTMI_REQUIRE(m >= 0 && n >= 0 && n < (1ll << 31), "bad shape");
+  TTMI_DISPATCH_FLOAT(dtype, T, return (layer_norm_dispatch<T, true>((T*)out, (const T*)input, (const T*)bias,
+                                                                      (const T*)gamma, (const T*)beta, m, n, eps,
+                                                                      (hipStream_t)stream, nullptr, nullptr, absmax_slots,
+                                                                      slots_written)));
   return 0;
 }
 

@@ -92,9 +92,17 @@ Tensor* Tensor::EnsureShadow() {
   return shadow_.get();
 }
 
+Tensor* Tensor::EnsureAbsmax() {
+  const DLTensor& t = dl();
+  if (!absmax_) absmax_.reset(new Tensor(nullptr));
+  absmax_->ReshapeAs(DataTypeTrait<float>::v, {TTMI_ABSMAX_SLOTS}, t.device.device_type, t.device.device_id, "absmax_slots");
+  return absmax_.get();
+}
+
 void* Tensor::ReshapeAs(DLDataType dtype, const std::vector<int64_t>& shape_list, DLDeviceType device_type,
                         int device_id, const std::string& name) {
   shadow_.reset();  // new contents: a producer that wants an fp32 copy calls EnsureShadow() afterwards
+  absmax_.reset();
   const size_t need = (size_t)Numel(shape_list) * (dtype.bits / 8);
   // Reuse only buffers allocated here (their shape storage and capacity are ours); tensors
   // imported from another framework are never resized in place.  A planned activation is looked up

@@ -71,6 +71,7 @@ class Tensor {
     DLManagedTensor* t = managed_;
     managed_ = nullptr;
     shadow_.reset();
+    absmax_.reset();
     return t;
   }
 
@@ -82,6 +83,13 @@ class Tensor {
   void DropShadow() { shadow_.reset(); }
   // Hand the fp32 copy to the caller (null when there is none); the tensor keeps its own buffer.
   std::unique_ptr<Tensor> TakeShadow() { return std::move(shadow_); }
+
+  // Optional per-workgroup maxima of |value| (TTMI_ABSMAX_SLOTS floats on the device), attached by the kernel that
+  // produced this tensor for the dynamic int8 quantisation of the Linear that consumes it (ttmi_*_absmax); like
+  // the fp32 copy it travels with the tensor and is dropped whenever the buffer is handed out or re-shaped.
+  const Tensor* absmax() const { return absmax_.get(); }
+  Tensor* EnsureAbsmax();
+  void DropAbsmax() { absmax_.reset(); }
 
   bool is_null() const { return managed_ == nullptr && !is_view_; }
 
@@ -127,10 +135,18 @@ class Tensor {
     return reinterpret_cast<const T*>(t.data);
   }
   template <typename T>
-  T* mutableData() { return const_cast<T*>(data<T>()); }
+  // (asking for a writable pointer drops the attached maxima: whoever writes the buffer invalidates them, and a
+  // producer that supplies new ones calls EnsureAbsmax() afterwards)
+  T* mutableData() {
+    absmax_.reset();
+    return const_cast<T*>(data<T>());
+  }
 
   const void* raw() const { return dl().data; }
-  void* mutable_raw() { return dl().data; }
+  void* mutable_raw() {
+    absmax_.reset();
+    return dl().data;
+  }
 
   // View of the n-th slice along dimension 0 (does not own memory).
   Tensor operator[](int64_t n);
@@ -147,9 +163,11 @@ class Tensor {
     managed_ = nullptr;
     is_view_ = false;
     shadow_.reset();
+    absmax_.reset();
   }
   void MoveFrom(Tensor& o) {
     shadow_ = std::move(o.shadow_);
+    absmax_ = std::move(o.absmax_);
     managed_ = o.managed_;
     is_view_ = o.is_view_;
     view_ = o.view_;
@@ -164,6 +182,7 @@ class Tensor {
   DLTensor view_{};
   std::vector<int64_t> view_shape_;
   std::unique_ptr<Tensor> shadow_;
+  std::unique_ptr<Tensor> absmax_;
 };
 
 // Copy `numel` elements between buffers on the stream; host<->device copies synchronise

@@ -227,7 +227,8 @@ void FusedAddBiasGELU::operator()(Tensor* output_tensor) const {
 }
 
 void FusedAddBiasLayerNorm::operator()(const Tensor& input_tensor, Tensor* output_tensor) const {
-  kernels::AddBiasLayerNorm<float>(input_tensor, dense_bias_, layer_norm_weight_, layer_norm_bias_, output_tensor, 1e-12f);
+  // (the quantized layers' epilogue: its result is what the next quantized Linear quantises)
+  kernels::AddBiasLayerNormWithAbsmax(input_tensor, dense_bias_, layer_norm_weight_, layer_norm_bias_, output_tensor, 1e-12f);
 }
 
 }  // namespace layers

@@ -197,6 +197,29 @@ void AddBiasLayerNorm(const Tensor& input_tensor, const Tensor& bias_tensor, con
 template void AddBiasLayerNorm<float>(const Tensor&, const Tensor&, const Tensor&, const Tensor&, Tensor*, float,
                                       const std::string);
 
+// AddBiasLayerNorm that also leaves the per-workgroup maxima of its result with the output tensor (fp32 tensors of
+// the quantized layers: the next Linear quantises this result and needs max|x| for its scale).
+void AddBiasLayerNormWithAbsmax(const Tensor& input_tensor, const Tensor& bias_tensor, const Tensor& gamma_tensor,
+                                const Tensor& beta_tensor, Tensor* out_tensor, float eps) {
+  RequireGpu(*out_tensor, "AddBiasLayerNorm");
+  if (core::ToDeviceDType(out_tensor->dtype()) != TTMI_F32) {
+    AddBiasLayerNorm<float>(input_tensor, bias_tensor, gamma_tensor, beta_tensor, out_tensor, eps);
+    return;
+  }
+  const int64_t n = input_tensor.shape(-1), m = input_tensor.numel() / n;
+  TT_ENFORCE_EQ(n, gamma_tensor.shape(0), "AddBiasLayerNorm input_tensor.shape(-1) should be the same as gamma_tensor.shape(0)");
+  TT_ENFORCE_EQ(n, beta_tensor.shape(0), "AddBiasLayerNorm input_tensor.shape(-1) should be the same as beta_tensor.shape(0)");
+  TT_ENFORCE_EQ(n, bias_tensor.shape(0), "AddBiasLayerNorm input_tensor.shape(-1) should be the same as bias_tensor.shape(0)");
+  TT_ENFORCE(common::is_same_shape(input_tensor, *out_tensor), "The shape of the input_tensor and out_tensor is not equal.");
+  RequireSameDType(input_tensor, *out_tensor, "AddBiasLayerNorm");
+  void* out = out_tensor->mutable_raw();
+  float* slots = out_tensor->EnsureAbsmax()->mutableData<float>();
+  int written = 0;
+  TT_DEVICE_CALL(ttmi_add_bias_layer_norm_absmax(out, input_tensor.raw(), bias_tensor.raw(), gamma_tensor.raw(), beta_tensor.raw(), m,
+                                                 n, eps, TTMI_F32, slots, &written, Stream()));
+  if (written == 0) out_tensor->DropAbsmax();
+}
+
 bool KeepsFp32Residual(const Tensor& t) { return core::ToDeviceDType(t.dtype()) == TTMI_BF16; }
 
 void AddBiasLayerNormResidual(const Tensor& input_tensor, const Tensor& bias_tensor, const Tensor& gamma_tensor,

@@ -85,6 +85,8 @@ void Transform(int64_t* src_data, float* dst_data, int64_t size, DLDeviceType de
 void AddBiasLayerNormResidual(const core::Tensor& input_tensor, const core::Tensor& bias_tensor,
                               const core::Tensor& gamma_tensor, const core::Tensor& beta_tensor, core::Tensor* out_tensor,
                               float eps = 1e-12f);
+void AddBiasLayerNormWithAbsmax(const core::Tensor& input_tensor, const core::Tensor& bias_tensor, const core::Tensor& gamma_tensor,
+                                const core::Tensor& beta_tensor, core::Tensor* out_tensor, float eps);
 bool KeepsFp32Residual(const core::Tensor& t);  // true for bfloat16 tensors
 // out = AddBiasLayerNorm(in . w^T, residual) with the same treatment of the residual; `w_nk` is the
 // [n, k] weight on the device, `out_tensor` already has its [.., n] shape.

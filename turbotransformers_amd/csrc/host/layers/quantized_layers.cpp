@@ -49,7 +49,13 @@ const int8_t* QuantizedLinear::QuantizeInput(const Tensor& input_tensor) const {
   TT_ENFORCE_EQ(input_tensor.shape(-1), k, "input width and weight rows differ");
   const int64_t m = input_tensor.numel() / k;
   int8_t* qx = q_input_.Reshape<int8_t>({m, k}, input_tensor.device_type(), input_tensor.device_id(), "QuantizedLinear/q_input");
-  TT_DEVICE_CALL(ttmi_quantize_rows_i8(input_tensor.data<float>(), qx, act_scale_.mutableData<float>(), m, k, Stream()));
+  if (input_tensor.absmax() != nullptr) {
+    // the kernel that produced the input left its per-workgroup maxima: one launch instead of two
+    TT_DEVICE_CALL(ttmi_quantize_rows_i8_from_absmax(input_tensor.data<float>(), qx, act_scale_.mutableData<float>(),
+                                                     input_tensor.absmax()->data<float>(), m, k, Stream()));
+  } else {
+    TT_DEVICE_CALL(ttmi_quantize_rows_i8(input_tensor.data<float>(), qx, act_scale_.mutableData<float>(), m, k, Stream()));
+  }
   return qx;
 }
 
@@ -60,9 +66,20 @@ void QuantizedLinear::operator()(const Tensor& input_tensor, Tensor* output_tens
   for (size_t i = 0; i + 1 < input_tensor.n_dim(); ++i) shape.push_back(input_tensor.shape((int)i));
   shape.push_back(n);
   float* out = output_tensor->Reshape<float>(shape, input_tensor.device_type(), input_tensor.device_id(), "QuantizedLinear/Reshape");
-  // int8 GEMM with the dequantisation folded into its store: the int32 accumulators stay on chip
-  TT_DEVICE_CALL(ttmi_gemm_i8_dequant(qx, q_weight_.data<int8_t>(), out, act_scale_.data<float>(), w_scales_.data<float>(),
-                                      bias_.is_null() ? nullptr : bias_.data<float>(), act_, m, n, k, k, k, n, Stream()));
+  // int8 GEMM with the dequantisation folded into its store: the int32 accumulators stay on chip.  It also leaves the
+  // per-workgroup maxima of its output with the tensor, for the Linear that quantises that output next.
+  // (not for a bare product: that is the form in front of a fused bias + LayerNorm, which supplies its own)
+  if (bias_.is_null() && act_ < 0) {
+    TT_DEVICE_CALL(ttmi_gemm_i8_dequant(qx, q_weight_.data<int8_t>(), out, act_scale_.data<float>(), w_scales_.data<float>(), nullptr,
+                                        act_, m, n, k, k, k, n, Stream()));
+    return;
+  }
+  float* slots = output_tensor->EnsureAbsmax()->mutableData<float>();
+  int written = 0;
+  TT_DEVICE_CALL(ttmi_gemm_i8_dequant_absmax(qx, q_weight_.data<int8_t>(), out, act_scale_.data<float>(), w_scales_.data<float>(),
+                                             bias_.is_null() ? nullptr : bias_.data<float>(), act_, m, n, k, k, k, n, slots,
+                                             &written, Stream()));
+  if (written == 0) output_tensor->DropAbsmax();
 }
 
 void QuantizedLinear::ProjectToHeads(const Tensor& input_tensor, const Tensor& bias, int64_t seq, int64_t heads, Tensor* q,
@@ -101,7 +118,7 @@ void QuantizedBertAttention::operator()(const Tensor& input_tensor, const Tensor
     TT_DEVICE_CALL(ttmi_fused_attention(q_.raw(), k_.raw(), v_.raw(), mask, merged_.mutable_raw(), nullptr, B, heads_, S, d, 0,
                                         1.0f / std::sqrt((float)d), TTMI_F32, Stream()));
     dense_(merged_, output);
-    kernels::AddBiasLayerNorm<float>(input_tensor, dense_bias_, ln_weight_, ln_bias_, output, 1e-12f);
+    kernels::AddBiasLayerNormWithAbsmax(input_tensor, dense_bias_, ln_weight_, ln_bias_, output, 1e-12f);
     return;
   }
   Tensor* score = attn != nullptr ? attn : &score_scratch_;
@@ -112,7 +129,7 @@ void QuantizedBertAttention::operator()(const Tensor& input_tensor, const Tensor
   kernels::BatchMatMul(*score, false, v_, false, 1.0f, &ctx_, 0.f);
   kernels::TransposeForScore(&merged_, ctx_);
   dense_(merged_, output);
-  kernels::AddBiasLayerNorm<float>(input_tensor, dense_bias_, ln_weight_, ln_bias_, output, 1e-12f);
+  kernels::AddBiasLayerNormWithAbsmax(input_tensor, dense_bias_, ln_weight_, ln_bias_, output, 1e-12f);
 }
 
 }  // namespace layers

@@ -226,8 +226,11 @@ template <int BN, int MF>
 constexpr int w4_strip_pitch() { return BN == 256 ? 256 : BN + 16; }  // bytes per staged row (BN/2 columns of 2 bytes)
 // AS = stages of the A operand's ring (B always has two).  With three, the epilogue strips hold 16 rows instead of 32
 // so that everything still fits the 160 KB of a CU.
-template <int BN, int MF, int AS = 2>
-constexpr int w4_lds_bytes() { return (AS * 256 + 2 * BN) * kRowBytes + 4 * (AS == 3 ? 16 : 32) * w4_strip_pitch<BN, MF>(); }
+// DIRECT: no strips at all (row-major outputs stored straight from the accumulator layout).
+template <int BN, int MF, int AS = 2, bool DIRECT = false>
+constexpr int w4_lds_bytes() {
+  return (AS * 256 + 2 * BN) * kRowBytes + (DIRECT ? 0 : 4 * (AS == 3 ? 16 : 32) * w4_strip_pitch<BN, MF>());
+}
 
 // What the kernel needs from an epilogue besides bias_ptr(): finish(x) applied to acc + bias in fp32, and
 // dest8(m, n), the address of the 16 bytes that hold columns n..n+7 of output row m.
@@ -242,8 +245,14 @@ constexpr int w4_lds_bytes() { return (AS * 256 + 2 * BN) * kRowBytes + 4 * (AS 
 // have landed, the activations of the step after it may still be in flight.  Global STORES return out of order with
 // loads, so the first barrier of a tile, which may still have the previous tile's stores in flight, waits for
 // everything.  Epilogues with a column pass keep two stages (their transposed unit needs the larger strip).
-template <typename T, int BN, int MF, typename Epi, int AS = 2>
+// DIRECT: a row-major 16-bit output leaves straight from the accumulator layout, without the trip through a strip: after
+// the pair swap a lane holds 16 contiguous bytes of one row and the four lanes that share a row 64 contiguous bytes
+// between them, so a store instruction writes sixteen 64-byte segments instead of four 256-byte ones, and the LDS
+// round trip and its waits are gone.  The launcher uses it for the 256-wide tile (measured 1 % faster on the whole
+// BERT-base forward there, level at 192 wide).
+template <typename T, int BN, int MF, typename Epi, int AS = 2, bool DIRECT = false>
 __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, const Epi epi) {
+  static_assert(!DIRECT || (LinearDest<Epi>::value && MF == 16), "direct stores: row-major 16-bit outputs, 16-wide blocks");
   static_assert(sizeof(T) == 2, "16-bit operands");
   static_assert(MF == 32 || MF == 16, "block sizes of the matrix instructions");
   static_assert(AS == 2 || (AS == 3 && MF == 16 && !HasColumnPass<Epi>::value), "three A stages: 16-wide blocks, row-major epilogues");
@@ -728,11 +737,18 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
 #pragma unroll
               for (int e = 0; e < 8; ++e) rounded[e] = from_float<T>(epi.finish(out[e]));
               packed[v] = __builtin_bit_cast(Quad, pack_chunk(rounded));
+              if constexpr (DIRECT) {
+                const int r = i * GROUP + (MF == 32 ? lrow : 16 * (v / (CB / 2)) + lrow);  // row inside the wavefront's 128
+                const int ncol = wn0 + unit_chunk(v) * 8;
+                if ((whole_rows || m0 + wm0 + r < m_lim) && (whole_width || n0 + ncol < n_lim))
+                  store_c(packed[v], (uint32_t)(wm0 + r) * ldc_bytes + (uint32_t)ncol * (uint32_t)sizeof(T),
+                          (uint32_t)m0 * ldc_bytes + (uint32_t)n0 * (uint32_t)sizeof(T));
+              }
             }
           }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (i > 0 && !StoresF32<Epi>::value) {
+        if (i > 0 && !StoresF32<Epi>::value && !DIRECT) {
           const int row0 = m0 + wm0 + (i - 1) * GROUP;
           if constexpr (StoresF32<Epi>::value) {
           } else if constexpr (LinearDest<Epi>::value) {
@@ -754,7 +770,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
           }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (i < GROUPS && !StoresF32<Epi>::value) {
+        if (i < GROUPS && !StoresF32<Epi>::value && !DIRECT) {
           // same wavefront, LDS operations complete in order: no barrier between the writes and the reads
 #pragma unroll
           for (int v = 0; v < NV; ++v) strip_write(strip_lds + (uint32_t)wr_off[v], packed[v]);
@@ -892,15 +908,20 @@ static bool w4_output_fits(const GemmArgs& g, int64_t ldc) {
 
 // split_col: a column (multiple of 8) at which a fresh tile has to start whatever BN is (0 = none).
 // Three A stages where they fit (192-wide tiles, row-major epilogues).  Switch TTMI_W4_A_STAGES = 2 keeps two.
+// (fp32 outputs never use the strips, so they have the room at either width)
 template <int BN, typename Epi>
-constexpr bool w4_three_stages_fit() { return BN == 192 && !HasColumnPass<Epi>::value; }
+constexpr bool w4_three_stages_fit() { return (BN == 192 && !HasColumnPass<Epi>::value) || StoresF32<Epi>::value; }
 
-template <typename T, int BN, typename Epi, int AS = 2>
+template <typename T, int BN, typename Epi, int AS = 2, bool DIRECT = false>
 static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s, int split_col = 0) {
-  if constexpr (AS == 2 && w4_three_stages_fit<BN, Epi>()) {
+  if constexpr (AS == 2 && !DIRECT && w4_three_stages_fit<BN, Epi>()) {
     if (kernel_switch(kSwitchW4AStages) != 2) return launch_w4<T, BN, Epi, 3>(g, epi, s, split_col);
   }
-  constexpr int LDS = w4_lds_bytes<BN, kW4Block, AS>();
+  // The 256-wide tile has no room for a third stage beside its strips; its row-major 16-bit outputs leave without them
+  // (measured: direct stores 1 % faster on the BERT-base forward than the strips at this width, level at 192; a third
+  // stage IN PLACE of the strips, which fills the 160 KB to the last byte, 4 % slower).
+  if constexpr (AS == 2 && !DIRECT && BN == 256 && LinearDest<Epi>::value) return launch_w4<T, BN, Epi, 2, true>(g, epi, s, split_col);
+  constexpr int LDS = w4_lds_bytes<BN, kW4Block, AS, DIRECT || StoresF32<Epi>::value>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
   if (describe_only(AS == 3 ? "dma3_agpr" : "dma_agpr", 4, 256, BN)) return 0;
   g.tiles_m = (g.m + 255) / 256;
@@ -911,7 +932,7 @@ static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s, int split_col = 
   TTMI_REQUIRE(tiles < (1ll << 30), "GEMM grid too large");
   // one persistent workgroup per CU (the LDS allows no second one), a multiple of the XCD count
   const unsigned grid = (unsigned)(std::min<int64_t>(ceil_div(tiles, kNumXcd), std::max(1, compute_units() / kNumXcd)) * kNumXcd);
-  auto kern = gemm_w4_kernel<T, BN, kW4Block, Epi, AS>;
+  auto kern = gemm_w4_kernel<T, BN, kW4Block, Epi, AS, DIRECT>;
   const int rc = allow_large_lds(reinterpret_cast<const void*>(kern), LDS);
   if (rc != 0) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kW4Threads), LDS, s, g, epi);

@@ -249,7 +249,7 @@ constexpr int w4_lds_bytes() {
 // the pair swap a lane holds 16 contiguous bytes of one row and the four lanes that share a row 64 contiguous bytes
 // between them, so a store instruction writes sixteen 64-byte segments instead of four 256-byte ones, and the LDS
 // round trip and its waits are gone.  The launcher uses it for the 256-wide tile (measured 1 % faster on the whole
-// BERT-base forward there, level at 192 wide).
+// BERT-base forward there, level at 192 wide), where the freed LDS also makes room for the third A stage.
 template <typename T, int BN, int MF, typename Epi, int AS = 2, bool DIRECT = false>
 __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, const Epi epi) {
   static_assert(!DIRECT || (LinearDest<Epi>::value && MF == 16), "direct stores: row-major 16-bit outputs, 16-wide blocks");
@@ -688,6 +688,8 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
           if (block_in_one_sequence) col_ptr[pass] += st_row[pass] * epi.dim;  // the lane's share of the row part
         }
       }
+      // direct stores: row lrow of a 16-row block, the lane's 16 bytes of a 64-byte run (unit_chunk(0) names them)
+      const uint32_t direct_voff = (uint32_t)lrow * ldc_bytes + (uint32_t)unit_chunk(0) * 16u;
       Quad landed[PASSES];  // first-class vectors: arrays of a struct type may end up in scratch memory
       // The matrix instructions are inline asm, so the compiler's hazard recogniser does not see that the accumulator
       // reads below depend on them: wait out the longest write-to-read distance of the matrix pipe here.
@@ -738,11 +740,13 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
               for (int e = 0; e < 8; ++e) rounded[e] = from_float<T>(epi.finish(out[e]));
               packed[v] = __builtin_bit_cast(Quad, pack_chunk(rounded));
               if constexpr (DIRECT) {
-                const int r = i * GROUP + (MF == 32 ? lrow : 16 * (v / (CB / 2)) + lrow);  // row inside the wavefront's 128
+                // one per-lane offset for all stores of the tile (the lane's row and its share of the column); the
+                // 16-row block goes into the scalar offset, the pair of block columns into the immediate
+                const int rblk = i * GROUP + 16 * (v / (CB / 2));  // first row of the unit's 16-row block inside the wavefront's 128
                 const int ncol = wn0 + unit_chunk(v) * 8;
-                if ((whole_rows || m0 + wm0 + r < m_lim) && (whole_width || n0 + ncol < n_lim))
-                  store_c(packed[v], (uint32_t)(wm0 + r) * ldc_bytes + (uint32_t)ncol * (uint32_t)sizeof(T),
-                          (uint32_t)m0 * ldc_bytes + (uint32_t)n0 * (uint32_t)sizeof(T));
+                if ((whole_rows || m0 + wm0 + rblk + lrow < m_lim) && (whole_width || n0 + ncol < n_lim))
+                  store_c(packed[v], direct_voff + (uint32_t)(v % (CB / 2)) * 64u,
+                          (uint32_t)(m0 + wm0 + rblk) * ldc_bytes + (uint32_t)(n0 + wn0) * (uint32_t)sizeof(T));
               }
             }
           }
@@ -917,10 +921,14 @@ static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s, int split_col = 
   if constexpr (AS == 2 && !DIRECT && w4_three_stages_fit<BN, Epi>()) {
     if (kernel_switch(kSwitchW4AStages) != 2) return launch_w4<T, BN, Epi, 3>(g, epi, s, split_col);
   }
-  // The 256-wide tile has no room for a third stage beside its strips; its row-major 16-bit outputs leave without them
-  // (measured: direct stores 1 % faster on the BERT-base forward than the strips at this width, level at 192; a third
-  // stage IN PLACE of the strips, which fills the 160 KB to the last byte, 4 % slower).
-  if constexpr (AS == 2 && !DIRECT && BN == 256 && LinearDest<Epi>::value) return launch_w4<T, BN, Epi, 2, true>(g, epi, s, split_col);
+  // The 256-wide tile has no room for a third stage beside its strips; its row-major 16-bit outputs leave without
+  // them (direct stores measured 1 % faster on the BERT-base forward than the strips at this width, level at 192), and
+  // the third stage then fills the 160 KB to the last byte (another 0.5 % on the BERT-base and BERT-large forwards,
+  // once the direct stores share one per-lane offset: with an offset per store this variant spilled and lost 4 %).
+  if constexpr (AS == 2 && !DIRECT && BN == 256 && LinearDest<Epi>::value) {
+    if (kernel_switch(kSwitchW4AStages) != 2) return launch_w4<T, BN, Epi, 3, true>(g, epi, s, split_col);
+    return launch_w4<T, BN, Epi, 2, true>(g, epi, s, split_col);
+  }
   constexpr int LDS = w4_lds_bytes<BN, kW4Block, AS, DIRECT || StoresF32<Epi>::value>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
   if (describe_only(AS == 3 ? "dma3_agpr" : "dma_agpr", 4, 256, BN)) return 0;

@@ -165,7 +165,7 @@ def run_smart_batch(steps, warmup):
 # Keyed by (kernel of the roofline pass, dtype, batch, seq) AND by the kernel variant the library reports for that
 # product (ttmi_gemm_describe): when the tile choice changes the record no longer applies and `traffic` is null.
 MEASURED_TRAFFIC = {
-    ("ffn1_gemm+bias+gelu", "f16", 64, 512): {"variant": "dma_agpr4w_256x256", "fetch_bytes": 123175 * 2.0 * 1024,
+    ("ffn1_gemm+bias+gelu", "f16", 64, 512): {"variant": "dma3_agpr4w_256x256", "fetch_bytes": 123162 * 2.0 * 1024,
                                               "write_bytes": 196608 * 1.0 * 1024},
 }
 

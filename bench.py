@@ -520,6 +520,9 @@ def run_ffn2_probe(iters=20, batch=64, seq=512, hidden=768, ffn=3072):
     ffn1 = lambda: capi.check(lib.ttmi_gemm_fused(P(x), P(w1), P(own), T, F, H, H, H, F, capi.EPI_BIAS_ACT, ctypes.byref(args), cdt, S()))
     ffn1()
     other = own.clone()
+    args_b = capi.EpilogueArgs()
+    args_b.bias = b1.data_ptr()
+    ffn1_b = lambda: capi.check(lib.ttmi_gemm_fused(P(x), P(w1), P(own), T, F, H, H, H, F, capi.EPI_BIAS, ctypes.byref(args_b), cdt, S()))
     ffn2 = lambda a: (lambda: capi.check(lib.ttmi_gemm(P(a), P(w2), P(out), T, H, F, F, F, H, 1, 1.0, 0.0, cdt, S())))
     ln = lambda: capi.check(lib.ttmi_add_bias_layer_norm(P(out), P(res), P(bh), P(gam), P(bh), T, H, 1e-12, cdt, S()))
     copy_src, copy_dst = torch.randn(64 << 20, device="cuda"), torch.empty(64 << 20, device="cuda")
@@ -543,7 +546,10 @@ def run_ffn2_probe(iters=20, batch=64, seq=512, hidden=768, ffn=3072):
              ("FFN1, FFN2 (own)", [ffn1, ffn2(own)]), ("FFN1, FFN2 (other)", [ffn1, ffn2(other)]),
              ("LayerNorm, FFN2 (other)", [ln, ffn2(other)]), ("copy, FFN2 (other)", [flush, ffn2(other)]),
              ("LayerNorm, FFN1, FFN2 (own), LayerNorm", [ln, ffn1, ffn2(own), ln]),
-             ("FFN2 (other), FFN2 (other)", [ffn2(other), ffn2(other)])]
+             ("FFN2 (other), FFN2 (other)", [ffn2(other), ffn2(other)]),
+             # what the GELU in FFN1's epilogue costs in layer order: the same sequence with a bias-only epilogue
+             ("FFN1 bias only", [ffn1_b]),
+             ("LayerNorm, FFN1 bias only, FFN2 (own), LayerNorm", [ln, ffn1_b, ffn2(own), ln])]
     t = {}
     out_lines = ["# The second FFN product inside the forward and alone (`python3 bench.py --ffn2-probe`)", "",
                  "fp16, %d x %d tokens; loops of %d passes of each sequence, us per pass (events around the whole loop)." % (batch, seq, iters), "",
@@ -552,7 +558,7 @@ def run_ffn2_probe(iters=20, batch=64, seq=512, hidden=768, ffn=3072):
         for name, fns in cases:
             t[name] = timed(fns)
     single = {"FFN2 (own)": t["FFN2 (other)"], "FFN2 (other)": t["FFN2 (other)"], "FFN1": t["FFN1"], "LayerNorm": t["LayerNorm"],
-              "copy": t["copy 2 x 256 MiB"]}
+              "copy": t["copy 2 x 256 MiB"], "FFN1 bias only": t["FFN1 bias only"]}
     for name, _ in cases:
         parts = [p.strip() for p in name.split(",")]
         if len(parts) == 1:
@@ -560,6 +566,9 @@ def run_ffn2_probe(iters=20, batch=64, seq=512, hidden=768, ffn=3072):
         else:
             alone = sum(single[p] for p in parts)
             out_lines.append("| %s | %.1f | %.1f | %+.1f |" % (name, t[name], alone, t[name] - alone))
+    out_lines += ["", "GELU in FFN1's epilogue: %.1f us alone in a loop, %.1f us in layer order." % (
+        t["FFN1"] - t["FFN1 bias only"],
+        t["LayerNorm, FFN1, FFN2 (own), LayerNorm"] - t["LayerNorm, FFN1 bias only, FFN2 (own), LayerNorm"])]
     print("\n".join(out_lines))
 
 

@@ -65,6 +65,8 @@ TTMI_API const char* ttmi_last_error(void);
  *   "TTMI_STATIC_SCRATCH_LIMIT"  bytes of its buffer ttmi_gemm_bias_layer_norm_static admits (to test its refusal);
  *   "TTMI_W4_A_STAGES"      2 = the one-wavefront-per-SIMD GEMM kernel keeps two LDS stages for the A operand
  *                           where it would take three;
+ *   "TTMI_W4_SPLITK"        0 = ttmi_gemm_bias_layer_norm never cuts a product along K on that kernel, n >= 2 = n
+ *                           slices for every product that can be cut that way;
  *   -1 = the launcher decides (the default).
  * Each switch starts from the environment variable of the same name, which is read once, at the first launch or
  * the first call of this function; later changes of the environment are not seen. */

@@ -275,6 +275,50 @@ def test_gemm_bias_layer_norm_fp32_residual(ttmi, oracle, dt, M, N, K):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,slices,fp32_residual", [(6275, 768, 3072, -1, False), (6275, 768, 3072, -1, True),
+                                                        (700, 384, 768, 3, False), (1, 8, 512, 2, False),
+                                                        (1300, 1000, 1024, 4, True), (520, 200, 256, 2, False)])
+def test_gemm_bias_layer_norm_k_slices_on_the_large_tile_kernel(ttmi, oracle, dt, M, N, K, slices, fp32_residual):
+    """The projection in front of a LayerNorm cut along K on the one-wavefront-per-SIMD kernel: (slice, tile) work
+    items, fp32 partial products, summed and normalised by the reduction kernel.  Once where the library chooses that
+    path by itself (the second FFN product of a 6275-token batch: 100 tiles for 256 CUs), and forced onto small and
+    ragged shapes with 2, 3 and 4 slices (switch TTMI_W4_SPLITK).  Against the oracle, and against the same call with
+    the path switched off: both sum fp32 partial sums of the same products, in another order."""
+    rng = np.random.default_rng(M + N + K)
+    A, W = _ab(rng, M, N, K, 1)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    bias, gamma, beta = (rng.standard_normal(N).astype(np.float32) for _ in range(3))
+    dA, dW = dev(A, dt), dev(W, dt)
+    dres = dev(res) if fp32_residual else dev(res, dt)
+    args = (ptr(dev(bias, dt)), ptr(dev(gamma, dt)), ptr(dev(beta, dt)))
+    outs = {}
+    try:
+        for name, value in (("sliced", slices), ("unsliced", 0)):
+            ok(ttmi.ttmi_set_kernel_switch(b"TTMI_W4_SPLITK", value))
+            out = torch.full((M + 8, N), -7.0, dtype=dA.dtype, device="cuda")
+            out32 = torch.full((M + 8, N), -7.0, device="cuda") if fp32_residual else None
+            ok(ttmi.ttmi_gemm_bias_layer_norm(ptr(dA), ptr(dW), ptr(out), None if fp32_residual else ptr(dres),
+                                              ptr(dres) if fp32_residual else None, *args,
+                                              ptr(out32) if fp32_residual else None, M, N, K, 1e-12, TTMI_DTYPES[dt], stream()))
+            torch.cuda.synchronize()
+            assert torch.all(out[M:] == -7.0), "rows past M were written"
+            outs[name] = (out[:M], out32[:M] if fp32_residual else None)
+    finally:
+        ok(ttmi.ttmi_set_kernel_switch(b"TTMI_W4_SPLITK", -1))
+    base = oracle.matmul(rounded(A, dt), rounded(W, dt), True)
+    want = oracle.add_bias_layer_norm(base, res if fp32_residual else rounded(res, dt), rounded(bias, dt), rounded(gamma, dt),
+                                      rounded(beta, dt))
+    got, got32 = outs["sliced"]
+    assert _ln_close(host(got), want, dt)
+    if fp32_residual:
+        assert _ln_close(host(got32), want, "f32")  # nothing rounded between the accumulators and the normalisation
+        assert np.array_equal(host(got), rounded(host(got32), dt))
+        assert max_abs(host(got32), host(outs["unsliced"][1])) < 1e-3
+    else:
+        assert _ln_close(host(got), host(outs["unsliced"][0]).astype(np.float32), dt)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
 @pytest.mark.parametrize("forced", [False, True])
 @pytest.mark.parametrize("M,N,K,with_bias", [(300, 200, 256, True), (4100, 1024, 1024, False), (2560, 768, 3072, True),
                                              (8192, 768, 768, True), (777, 776, 384, False), (128, 768, 3072, True)])

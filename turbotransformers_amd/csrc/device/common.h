@@ -42,7 +42,7 @@ int* async_error_flag();  // device-visible pinned int, 0 = ok
 // from an environment variable read ONCE (first use; a launch never scans the environment) and can be changed
 // afterwards through ttmi_set_kernel_switch.  kSwitchUnset = the launcher decides.
 constexpr int kSwitchUnset = -1;
-enum KernelSwitch { kSwitchLargeTile = 0, kSwitchWaveKernel = 1, kSwitchAttentionWaves = 2, kSwitchStaticScratchLimit = 3, kSwitchW4AStages = 4, kNumKernelSwitches = 5 };
+enum KernelSwitch { kSwitchLargeTile = 0, kSwitchWaveKernel = 1, kSwitchAttentionWaves = 2, kSwitchStaticScratchLimit = 3, kSwitchW4AStages = 4, kSwitchW4SplitK = 5, kNumKernelSwitches = 6 };
 int kernel_switch(KernelSwitch which);
 
 // ---- scalar conversion ----------------------------------------------------------------

@@ -53,13 +53,17 @@ static int gemm_bias_layer_norm_impl(const void* a, const void* w, void* out, co
                          aligned_rows(gamma, sizeof(T)) && aligned_rows(beta, sizeof(T)) &&
                          (residual_f32 != nullptr ? aligned16(residual_f32) && aligned16(out_f32) : aligned_rows(residual, sizeof(T)));
     const SplitPlan plan = rows_ok ? plan_split<T>(m, n, k, 1, aligned) : SplitPlan{SplitKind::kNone, 1};
-    if (plan.kind != SplitKind::kNone) {
-      GemmArgs g{};
-      g.a = (const char*)a;
-      g.b = (const char*)w;
-      g.m = (int)m; g.n = (int)n; g.k = (int)k;
-      g.lda = k; g.ldb = k;
-      g.inner = 1;
+    GemmArgs g{};
+    g.a = (const char*)a;
+    g.b = (const char*)w;
+    g.m = (int)m; g.n = (int)n; g.k = (int)k;
+    g.lda = k; g.ldb = k;
+    g.inner = 1;
+    int large_tile_slices = 0;
+    if constexpr (sizeof(T) == 2) {
+      if (rows_ok) large_tile_slices = w4_splitk_slices<T>(g, aligned);
+    }
+    if (plan.kind != SplitKind::kNone || large_tile_slices > 1) {
       auto reduce = [&](const float* ws, int slices, bool, hipStream_t st) {
         auto launch = [&](auto iters) {
           hipLaunchKernelGGL((splitk_reduce_layer_norm_kernel<T, decltype(iters)::value>), dim3((unsigned)m), dim3(256), 0, st, ws,
@@ -71,6 +75,9 @@ static int gemm_bias_layer_norm_impl(const void* a, const void* w, void* out, co
         else launch(std::integral_constant<int, 4>{});
       };
       constexpr int BK = kRowBytes / sizeof(T);
+      if constexpr (sizeof(T) == 2) {
+        if (large_tile_slices > 1) return (launch_w4_splitk<T>(g, large_tile_slices, s, reduce));
+      }
       if (plan.kind == SplitKind::kDmaTiles) return (launch_fast_splitk<T>(g, plan.splits, k / BK, BK, s, reduce));
       return (launch_splitk<T>(g, plan.splits, k / BK, BK, s, reduce));
     }

@@ -276,14 +276,34 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   extern __shared__ __align__(16) char smem[];
 
   // Tiles of this workgroup: XCD x owns [x*per_xcd, (x+1)*per_xcd); its workgroups stride through it together.
-  const int tiles = g.tiles_m * g.tiles_n;
+  // K slices (fp32 outputs only): with g.k_chunk > 0 the work items are (slice, tile) pairs, slice-major; slice z
+  // multiplies columns [z*k_chunk, (z+1)*k_chunk) of both operands and stores its partial product as rows
+  // [z*M, (z+1)*M) of the output, for a reduction pass to sum.
+  const int tiles_mn = g.tiles_m * g.tiles_n;
+  int slices = 1;
+  if constexpr (StoresF32<Epi>::value) {
+    if (g.k_chunk > 0) slices = g.k / g.k_chunk;
+  }
+  const int tiles = tiles_mn * slices;
+  auto locate = [&](int item, int& tile_m, int& tile_n) __attribute__((always_inline)) {
+    int z = 0;
+    if constexpr (StoresF32<Epi>::value) {
+      if (slices > 1) {
+        z = item / tiles_mn;
+        item -= z * tiles_mn;
+      }
+    }
+    tile_coords(item, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    return z;
+  };
   const int per_xcd = (tiles + kNumXcd - 1) / kNumXcd;
   const int xcd = (int)(blockIdx.x % kNumXcd), stride = (int)(gridDim.x / kNumXcd);
   const int xcd_end = min((xcd + 1) * per_xcd, tiles);
   const int first = xcd * per_xcd + (int)(blockIdx.x / kNumXcd);
   if (first >= xcd_end) return;
   const int my_tiles = (xcd_end - first + stride - 1) / stride;
-  const int ksteps = g.k / BK;  // even (checked by the launcher)
+  const int ksteps = (slices > 1 ? g.k_chunk : g.k) / BK;  // even (checked by the launcher)
+  const uint32_t slice_bytes = (uint32_t)g.k_chunk * (uint32_t)sizeof(T);  // K offset of slice 1 inside an operand row
   const int total_steps = my_tiles * ksteps;
 
   const int64_t lda_bytes = g.lda * (int64_t)sizeof(T), ldb_bytes = g.ldb * (int64_t)sizeof(T);
@@ -311,7 +331,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   uint32_t a_soff = 0, b_soff = 0;  // byte offset of the cursor's tile in A and in B (matrices below 2 GiB, checked by the launcher)
   auto dma_point = [&](int tile) __attribute__((always_inline)) {
     int tile_m, tile_n;
-    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int z = locate(tile, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = first_column(tile_n);
     const int sub = lane >> 3, p = lane & 7;
 #pragma unroll
@@ -324,8 +344,8 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       const int row = (wave * B_LOADS + i) * 8 + sub;
       vob[i] = (uint32_t)(min(n0 + row, g.n - 1) - n0) * (uint32_t)ldb_bytes + ((p ^ ((row >> 1) & 7)) << 4);
     }
-    a_soff = (uint32_t)m0 * (uint32_t)lda_bytes;
-    b_soff = (uint32_t)n0 * (uint32_t)ldb_bytes;
+    a_soff = (uint32_t)m0 * (uint32_t)lda_bytes + (uint32_t)z * slice_bytes;
+    b_soff = (uint32_t)n0 * (uint32_t)ldb_bytes + (uint32_t)z * slice_bytes;
   };
   // load i of K step `dma_step` into stage dma_step & 1
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -375,7 +395,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   int b_step = 0, b_k = 0, b_tile = first;
   auto a_point = [&](int tile) __attribute__((always_inline)) {
     int tile_m, tile_n;
-    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int z = locate(tile, tile_m, tile_n);
     const int m0 = tile_m * BM;
     const int sub = lane >> 3, p = lane & 7;
 #pragma unroll
@@ -383,11 +403,11 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       const int row = (wave * A_LOADS + i) * 8 + sub;
       voa[i] = (uint32_t)(min(m0 + row, g.m - 1) - m0) * (uint32_t)lda_bytes + ((p ^ ((row >> 1) & 7)) << 4);
     }
-    a_soff = (uint32_t)m0 * (uint32_t)lda_bytes;
+    a_soff = (uint32_t)m0 * (uint32_t)lda_bytes + (uint32_t)z * slice_bytes;
   };
   auto b_point = [&](int tile) __attribute__((always_inline)) {
     int tile_m, tile_n;
-    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int z = locate(tile, tile_m, tile_n);
     const int n0 = first_column(tile_n);
     const int sub = lane >> 3, p = lane & 7;
 #pragma unroll
@@ -395,7 +415,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       const int row = (wave * B_LOADS + i) * 8 + sub;
       vob[i] = (uint32_t)(min(n0 + row, g.n - 1) - n0) * (uint32_t)ldb_bytes + ((p ^ ((row >> 1) & 7)) << 4);
     }
-    b_soff = (uint32_t)n0 * (uint32_t)ldb_bytes;
+    b_soff = (uint32_t)n0 * (uint32_t)ldb_bytes + (uint32_t)z * slice_bytes;
   };
 #if defined(__HIP_DEVICE_COMPILE__)
   // load i of the split cursors: 0 .. B_LOADS-1 are the B loads (issued first), the rest the A loads
@@ -578,7 +598,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   int tile = first;
   for (int t = 0; t < my_tiles; ++t, tile += stride) {
     int tile_m, tile_n;
-    tile_coords(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int slice = locate(tile, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = first_column(tile_n);
     bool swap = true;
     if constexpr (HasColumnPass<Epi>::value) swap = !(epi.column_pass() && n0 >= epi.first_column_of_pass());
@@ -729,7 +749,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
               const int m = m0 + wm0 + i * GROUP + (MF == 32 ? lrow : 16 * (v / (CB / 2)) + lrow);
               const int ncol = n0 + wn0 + unit_chunk(v) * 8;
               if ((whole_rows || m < m_lim) && (whole_width || ncol < n_lim)) {
-                float* dst = epi.c + (int64_t)m * epi.ldc + ncol;
+                float* dst = epi.c + ((int64_t)slice * g.m + m) * epi.ldc + ncol;
                 *reinterpret_cast<floatx4*>(dst) = floatx4{out[0], out[1], out[2], out[3]};
                 *reinterpret_cast<floatx4*>(dst + 4) = floatx4{out[4], out[5], out[6], out[7]};
               }
@@ -931,12 +951,13 @@ static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s, int split_col = 
   }
   constexpr int LDS = w4_lds_bytes<BN, kW4Block, AS, DIRECT || StoresF32<Epi>::value>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
-  if (describe_only(AS == 3 ? "dma3_agpr" : "dma_agpr", 4, 256, BN)) return 0;
+  const int slices = g.k_chunk > 0 ? g.k / g.k_chunk : 1;  // K slices: fp32 outputs only (launch_w4_splitk)
+  if (describe_only(AS == 3 ? "dma3_agpr" : "dma_agpr", 4, 256, BN, slices)) return 0;
   g.tiles_m = (g.m + 255) / 256;
   g.split_col = split_col;
   g.split_tiles = split_col > 0 ? (split_col + BN - 1) / BN : 0;
   g.tiles_n = g.split_tiles + (g.n - split_col + BN - 1) / BN;
-  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * slices;
   TTMI_REQUIRE(tiles < (1ll << 30), "GEMM grid too large");
   // one persistent workgroup per CU (the LDS allows no second one), a multiple of the XCD count
   const unsigned grid = (unsigned)(std::min<int64_t>(ceil_div(tiles, kNumXcd), std::max(1, compute_units() / kNumXcd)) * kNumXcd);
@@ -974,6 +995,50 @@ template <typename T, typename Epi>
 static int launch_w4_linear(const GemmArgs& g, const Epi& epi, hipStream_t s) {
   if (tile_cost(kW4Tile256, g.m, g.n, 1) < tile_cost(kW4Tile192, g.m, g.n, 1)) return launch_w4<T, 256>(g, epi, s);
   return launch_w4<T, 192>(g, epi, s);
+}
+
+// A product cut along K on this kernel: the work items are (slice, tile) pairs, every slice leaves its partial product
+// in fp32 (rows [z*M, (z+1)*M) of the workspace) and `reduce(ws, slices, vec, stream)` sums them and applies the
+// epilogue.  For a few thousand rows by a narrow output and a long K (the second FFN product of a 20-request batch:
+// 6275 x 768 x 3072), where whole tiles are too few for the CUs whatever their size: 100 tiles of 256 x 192 with 48 K
+// steps each become 200 items of 24 steps.  Every slice has the same, even number of K steps.
+template <typename T>
+static bool w4_splitk_ok(const GemmArgs& g, int splits, bool aligned) {
+  constexpr int BK = kRowBytes / (int)sizeof(T);
+  return splits > 1 && w4_eligible<T>(g, 1, aligned) && g.k % (splits * 2 * BK) == 0 && g.n % 8 == 0 &&
+         (int64_t)splits * g.m * g.n * 4 < ((int64_t)1 << 31);
+}
+// How many K slices such a product gets on this kernel (0 or 1 = it is not taken).  Switch TTMI_W4_SPLITK: 0 = never,
+// n >= 2 = n slices for every product that can be cut that way.
+template <typename T>
+static int w4_splitk_slices(const GemmArgs& g, bool aligned) {
+  const int force = kernel_switch(kSwitchW4SplitK);
+  if (force == 0 || kernel_switch(kSwitchLargeTile) == 0) return 0;
+  if (force >= 2) return w4_splitk_ok<T>(g, force, aligned) ? force : 0;
+  // Two slices where they turn 0.35-0.5 rounds of whole tiles into 0.7-1 round of items and K is long enough to
+  // pay for the fp32 partial products (measured, LayerNorm included: 6275 x 768 x 3072 54 -> 46 us; at 4924 and at
+  // 10000 rows, where the 8-wavefront kernels' own tiles fill the chip better, level, and not taken).
+  constexpr int BK = kRowBytes / (int)sizeof(T);
+  if (g.k / BK < 32 || !w4_splitk_ok<T>(g, 2, aligned)) return 0;
+  const bool wide = tile_cost(kW4Tile256, g.m, g.n, 2) < tile_cost(kW4Tile192, g.m, g.n, 2);  // as launch_w4_splitk picks
+  const int64_t tiles = ceil_div(g.m, 256) * ceil_div(g.n, wide ? 256 : 192);
+  const int64_t cus = compute_units();
+  return (2 * tiles <= cus && 2 * tiles * 10 > cus * 7) ? 2 : 0;
+}
+template <typename T, typename Reduce>
+static int launch_w4_splitk(GemmArgs g, int splits, hipStream_t s, const Reduce& reduce) {
+  float* ws = nullptr;
+  if (tl_describe == nullptr) {
+    const int rc = splitk_workspace((size_t)splits * g.m * g.n * sizeof(float), s, &ws);
+    if (rc != 0) return rc;
+  }
+  g.k_chunk = g.k / splits;
+  const EpiF32<T> part{ws, nullptr, g.n, true};
+  const int rc = tile_cost(kW4Tile256, g.m, g.n, splits) < tile_cost(kW4Tile192, g.m, g.n, splits) ? launch_w4<T, 256>(g, part, s)
+                                                                                                  : launch_w4<T, 192>(g, part, s);
+  if (rc != 0 || tl_describe != nullptr) return rc;
+  reduce(ws, splits, true, s);
+  return launch_status("gemm_w4_splitk");
 }
 
 // Bias, and bias + activation.  With an activation the epilogue is a long stretch of VALU work (two transcendentals

@@ -10,7 +10,7 @@ namespace ttmi {
 
 namespace {
 const char* const kSwitchNames[kNumKernelSwitches] = {"TTMI_LARGE_TILE", "TTMI_WAVE_KERNEL", "TTMI_ATTENTION_WAVES",
-                                                       "TTMI_STATIC_SCRATCH_LIMIT", "TTMI_W4_A_STAGES"};
+                                                       "TTMI_STATIC_SCRATCH_LIMIT", "TTMI_W4_A_STAGES", "TTMI_W4_SPLITK"};
 struct KernelSwitches {
   std::atomic<int> value[kNumKernelSwitches];
   KernelSwitches() {

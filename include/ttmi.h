@@ -398,6 +398,8 @@ TTMI_API int ttmi_yardstick_mfma(int block, int dtype, const void* operands, int
  *                  them (then the slots are untouched and the consumer calls ttmi_quantize_rows_i8 as before).
  * ttmi_add_bias_layer_norm_absmax   = ttmi_add_bias_layer_norm, the same bits in `out`;
  * ttmi_gemm_i8_dequant_absmax       = ttmi_gemm_i8_dequant, the same bits in `c` (maximum taken after the activation);
+ * ttmi_fused_attention_absmax       = ttmi_fused_attention, the same bits in `out`; the maxima are left by dense
+ *                                     fp32 launches only (any other call reports 0 slots written);
  * ttmi_quantize_rows_i8_from_absmax = the second half of ttmi_quantize_rows_i8: scale from the slots' maximum,
  *                                     scale_dev[0] / [1] as there, the same bits in `q`.
  * No counterpart in the reference, whose quantized Linear is its framework's dynamic quantisation
@@ -406,6 +408,10 @@ TTMI_API int ttmi_yardstick_mfma(int block, int dtype, const void* operands, int
 TTMI_API int ttmi_add_bias_layer_norm_absmax(void* out, const void* input, const void* bias, const void* gamma,
                                              const void* beta, int64_t m, int64_t n, float eps, int dtype,
                                              float* absmax_slots, int* slots_written, void* stream);
+TTMI_API int ttmi_fused_attention_absmax(const void* q, const void* k, const void* v, const float* mask, void* out,
+                                         const int32_t* cu_seqlens, int64_t batch, int64_t heads, int64_t seq,
+                                         int64_t head_dim, int64_t v_seq_pitch, float scale, int dtype,
+                                         float* absmax_slots, int* slots_written, void* stream);
 TTMI_API int ttmi_gemm_i8_dequant_absmax(const int8_t* a, const int8_t* b, float* c, const float* act_scale_dev,
                                          const float* w_scale, const float* bias, int act, int64_t m, int64_t n,
                                          int64_t k, int64_t lda, int64_t ldb, int64_t ldc, float* absmax_slots,

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import ALL_DTYPES, TTMI_DTYPES, dev, host, max_abs, ok, ptr, rounded, stream
+from helpers import ALL_DTYPES, TORCH_DTYPES, TTMI_DTYPES, dev, host, max_abs, ok, ptr, rounded, stream
 from turbotransformers_amd import capi
 
 pytestmark = pytest.mark.gpu
@@ -742,6 +742,41 @@ def test_fused_attention_fp32_vs_unfused_oracle(ttmi, oracle, attention_waves, B
     prob = oracle.apply_mask_and_softmax(score, mask, 1.0, True)
     want = oracle.transpose_for_score(oracle.batch_matmul(prob, V, False)).reshape(B, S, h * d)
     assert max_abs(host(out), want) <= 5e-5
+    # the form that also leaves the per-workgroup maxima of its output (for the int8 Linear that quantises it next):
+    # the same bits, every slot written, their maximum is max|out|
+    import ctypes
+    out2 = torch.full((B, S, h * d), 9.0, dtype=torch.float32, device="cuda")
+    slots = torch.full((capi.ABSMAX_SLOTS, ), float("nan"), device="cuda")
+    written = ctypes.c_int(-1)
+    ok(ttmi.ttmi_fused_attention_absmax(ptr(dQ), ptr(dK), ptr(dV), ptr(dev(mask)) if masked else None, ptr(out2), None, B, h, S,
+                                        d, pitch, 0.125, TTMI_DTYPES["f32"], ptr(slots), ctypes.byref(written), stream()))
+    assert torch.equal(out, out2)
+    assert written.value == capi.ABSMAX_SLOTS and not torch.isnan(slots).any()
+    assert float(slots.max()) == float(out.abs().max())
+
+
+def test_fused_attention_absmax_reports_no_slots_where_it_leaves_none(ttmi):
+    """16-bit types, packed batches and launches with more workgroups than slots: the output as always, 0 slots
+    reported, the slots untouched."""
+    import ctypes
+    d = 64
+    for dt, B, h, S, packed in (("f16", 2, 2, 64, False), ("f32", 2, 2, 64, True), ("f32", 90, 12, 32, False)):
+        g = torch.Generator(device="cuda").manual_seed(S + B)
+        q, k, v = (torch.randn((B, h, S, d), device="cuda", generator=g).to(TORCH_DTYPES[dt]) for _ in range(3))
+        cu = torch.arange(0, (B + 1) * S, S, dtype=torch.int32, device="cuda") if packed else None
+        outs = []
+        for with_slots in (False, True):
+            out = torch.zeros((B, S, h * d), dtype=q.dtype, device="cuda")
+            slots = torch.full((capi.ABSMAX_SLOTS, ), float("nan"), device="cuda")
+            written = ctypes.c_int(-1)
+            args = (ptr(q), ptr(k), ptr(v), None, ptr(out), ptr(cu) if packed else None, B, h, S, d, 0, 0.125, TTMI_DTYPES[dt])
+            if with_slots:
+                ok(ttmi.ttmi_fused_attention_absmax(*args, ptr(slots), ctypes.byref(written), stream()))
+                assert written.value == 0 and torch.isnan(slots).all()
+            else:
+                ok(ttmi.ttmi_fused_attention(*args, stream()))
+            outs.append(out)
+        assert torch.equal(outs[0], outs[1])
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])

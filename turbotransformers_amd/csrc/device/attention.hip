@@ -346,16 +346,13 @@ __global__ __launch_bounds__(NW * 64, 16 / NW) void fused_attention_kernel(const
 namespace ttmi {
 // attention_f32.hip: the fp32 form
 int fused_attention_f32(const float* q, const float* k, const float* v, const float* mask, float* out, const int32_t* cu,
-                        int64_t batch, int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, hipStream_t s);
-}  // namespace ttmi
+                        int64_t batch, int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, float* absmax,
+                        hipStream_t s);
 
-using namespace ttmi;
-
-extern "C" {
-
-int ttmi_fused_attention(const void* q, const void* k, const void* v, const float* mask, void* out,
-                         const int32_t* cu_seqlens, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
-                         int64_t v_seq_pitch, float scale, int dtype, void* stream) {
+// absmax / slots_written: see ttmi_fused_attention_absmax; both null for the plain entry point
+static int fused_attention_impl(const void* q, const void* k, const void* v, const float* mask, void* out,
+                                const int32_t* cu_seqlens, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
+                                int64_t v_seq_pitch, float scale, int dtype, float* absmax, int* slots_written, void* stream) {
   TTMI_REQUIRE(q && k && v && out, "null tensor");
   TTMI_REQUIRE(head_dim == kD, "fused attention is built for head_dim 64");
   TTMI_REQUIRE(dtype == TTMI_F16 || dtype == TTMI_BF16 || dtype == TTMI_F32, "fused attention is built for fp16 / bf16 / fp32");
@@ -385,9 +382,14 @@ int ttmi_fused_attention(const void* q, const void* k, const void* v, const floa
   const dim3 grid((unsigned)ceil_div(seq, nw * 32), (unsigned)(batch * heads));
   const float sl2 = scale * 1.4426950408889634f, inv_scale = 1.0f / scale;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == TTMI_F32)
-    return fused_attention_f32((const float*)q, (const float*)k, (const float*)v, mask, (float*)out, cu_seqlens, batch, heads,
-                               seq, v_seq_pitch, scale, nw, s);
+  if (dtype == TTMI_F32) {
+    // the per-workgroup maxima: dense fp32 batches whose workgroups fit the slots
+    const bool leave_maxima = absmax != nullptr && cu_seqlens == nullptr && (int64_t)grid.x * grid.y <= TTMI_ABSMAX_SLOTS;
+    const int rc = fused_attention_f32((const float*)q, (const float*)k, (const float*)v, mask, (float*)out, cu_seqlens, batch,
+                                       heads, seq, v_seq_pitch, scale, nw, leave_maxima ? absmax : nullptr, s);
+    if (rc == 0 && leave_maxima && slots_written != nullptr) *slots_written = TTMI_ABSMAX_SLOTS;
+    return rc;
+  }
 #define TTMI_FA_LAUNCH(T, PACKED, VT, NW)                                                                              \
   hipLaunchKernelGGL((fused_attention_kernel<T, PACKED, VT, NW>), grid, dim3(NW * 64), 0, s, (const T*)q, (const T*)k, \
                      (const T*)v, mask, (T*)out, cu_seqlens, (int)heads, (int)seq, (int)v_seq_pitch, sl2, inv_scale)
@@ -410,6 +412,28 @@ int ttmi_fused_attention(const void* q, const void* k, const void* v, const floa
 #undef TTMI_FA_WAVES
 #undef TTMI_FA_LAUNCH
   return launch_status("fused_attention");
+}
+}  // namespace ttmi
+
+using namespace ttmi;
+
+extern "C" {
+
+int ttmi_fused_attention(const void* q, const void* k, const void* v, const float* mask, void* out,
+                         const int32_t* cu_seqlens, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
+                         int64_t v_seq_pitch, float scale, int dtype, void* stream) {
+  return fused_attention_impl(q, k, v, mask, out, cu_seqlens, batch, heads, seq, head_dim, v_seq_pitch, scale, dtype, nullptr,
+                              nullptr, stream);
+}
+
+int ttmi_fused_attention_absmax(const void* q, const void* k, const void* v, const float* mask, void* out,
+                                const int32_t* cu_seqlens, int64_t batch, int64_t heads, int64_t seq, int64_t head_dim,
+                                int64_t v_seq_pitch, float scale, int dtype, float* absmax_slots, int* slots_written,
+                                void* stream) {
+  TTMI_REQUIRE(absmax_slots && slots_written, "null absmax arguments");
+  *slots_written = 0;
+  return fused_attention_impl(q, k, v, mask, out, cu_seqlens, batch, heads, seq, head_dim, v_seq_pitch, scale, dtype,
+                              absmax_slots, slots_written, stream);
 }
 
 }  // extern "C"

@@ -59,7 +59,7 @@ template <int NW, bool VT, bool PACKED>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void fused_attention_f32_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ mask,
     float* __restrict__ out, const int32_t* __restrict__ cu, int heads, int seq, int v_pitch, float scale_log2e,
-    float inv_scale) {
+    float inv_scale, float* __restrict__ absmax) {
   static_assert(NW == 4 || NW == 8, "four or eight wavefronts");
   constexpr int kBQ = NW * 32;               // queries per workgroup
   constexpr int kPieces = 1024 / (NW * 64);  // 16-byte pieces of a K (V^T) tile per thread: 64 rows of 16
@@ -242,6 +242,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
       *reinterpret_cast<floatx4*>(stage_o + lrow * (kD + 4) + t * 32 + 8 * g + 4 * lhalf) = c;
     }
   const int hd = heads * kD;
+  float amax = 0.f;
 #pragma unroll
   for (int p = 0; p < 8; ++p) {
     const int r = p * 4 + (lane >> 4), cchunk = lane & 15;
@@ -249,7 +250,26 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     if (qi < q_len) {
       const floatx4 x = *reinterpret_cast<const floatx4*>(stage_o + r * (kD + 4) + cchunk * 4);
       *reinterpret_cast<floatx4*>(out + ((int64_t)out_row0 + qi) * hd + head * kD + cchunk * 4) = x;
+      amax = fmaxf(fmaxf(amax, fmaxf(fabsf(x[0]), fabsf(x[1]))), fmaxf(fabsf(x[2]), fabsf(x[3])));
     }
+  }
+  // Optional (dense batches): max|out| of this workgroup to its slot, for the int8 Linear that quantises `out` next;
+  // workgroup 0 zeroes the slots no workgroup owns, so every slot is written by every launch.
+  if (absmax != nullptr) {
+    amax = group_max<kWave>(amax);
+    __syncthreads();  // every wavefront is done with its share of the output stage
+    float* red = reinterpret_cast<float*>(smem);
+    if (lane == 0) red[wave] = amax;
+    __syncthreads();
+    const int wg = (int)(blockIdx.y * gridDim.x + blockIdx.x), wgs = (int)(gridDim.x * gridDim.y);
+    if (tid == 0) {
+      float m = red[0];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) m = fmaxf(m, red[w]);
+      absmax[wg] = m;
+    }
+    if (wg == 0)
+      for (int i = wgs + tid; i < TTMI_ABSMAX_SLOTS; i += NW * 64) absmax[i] = 0.f;
   }
 }
 
@@ -257,7 +277,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
 
 // Launch; arguments were checked by ttmi_fused_attention.
 int fused_attention_f32(const float* q, const float* k, const float* v, const float* mask, float* out, const int32_t* cu,
-                        int64_t batch, int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, hipStream_t s) {
+                        int64_t batch, int64_t heads, int64_t seq, int64_t v_seq_pitch, float scale, int nw, float* absmax,
+                        hipStream_t s) {
   const dim3 grid((unsigned)ceil_div(seq, nw * 32), (unsigned)(batch * heads));
   const float sl2 = scale * 1.4426950408889634f, inv_scale = 1.0f / scale;
   // more than 64 KB of dynamic LDS: the limit is raised once per kernel and device
@@ -275,7 +296,7 @@ int fused_attention_f32(const float* q, const float* k, const float* v, const fl
       }
     }
     hipLaunchKernelGGL(kern, grid, dim3(threads), lds, s, q, k, v, mask, out, cu, (int)heads, (int)seq, (int)v_seq_pitch, sl2,
-                       inv_scale);
+                       inv_scale, absmax);
     return 0;
   };
   const bool vt = v_seq_pitch > 0, packed = cu != nullptr;

@@ -115,8 +115,13 @@ void QuantizedBertAttention::operator()(const Tensor& input_tensor, const Tensor
       TT_ENFORCE_EQ(attention_mask.numel(), B * S, "attention mask has the wrong size");
       mask = attention_mask.data<float>();
     }
-    TT_DEVICE_CALL(ttmi_fused_attention(q_.raw(), k_.raw(), v_.raw(), mask, merged_.mutable_raw(), nullptr, B, heads_, S, d, 0,
-                                        1.0f / std::sqrt((float)d), TTMI_F32, Stream()));
+    // the kernel leaves the maxima of the context with the tensor: the output projection quantises it in one launch
+    void* merged = merged_.mutable_raw();
+    float* slots = merged_.EnsureAbsmax()->mutableData<float>();
+    int written = 0;
+    TT_DEVICE_CALL(ttmi_fused_attention_absmax(q_.raw(), k_.raw(), v_.raw(), mask, merged, nullptr, B, heads_, S, d, 0,
+                                               1.0f / std::sqrt((float)d), TTMI_F32, slots, &written, Stream()));
+    if (written == 0) merged_.DropAbsmax();
     dense_(merged_, output);
     kernels::AddBiasLayerNormWithAbsmax(input_tensor, dense_bias_, ln_weight_, ln_bias_, output, 1e-12f);
     return;

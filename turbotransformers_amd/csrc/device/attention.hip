@@ -99,6 +99,104 @@ __device__ __forceinline__ int vt_pos(int within16) {
   return (within16 & 3) | ((within16 & 4) << 1) | ((within16 & 8) >> 1);
 }
 
+// One 64-key tile: kt = K tile ([key][d], 128-byte rows, swizzled), vt = V^T tile ([d][key], likewise), mk = additive
+// mask of its 64 keys divided by the score scale.  m_run is kept in raw score units; the softmax scale and log2(e)
+// are applied inside the exp2 argument: p = exp2(s*c - m*c), c = scale*log2(e).  k_off: the lane's four fragment
+// offsets inside a 32-row block (see the kernels).
+template <typename T>
+__device__ __forceinline__ void attention_tile(const char* kt, const char* vt, const float* mk, const Chunk16 (&qf)[4],
+                                               const int (&k_off)[4], int lhalf, float scale_log2e, floatx16 (&ot)[2],
+                                               float& m_run, float& l_run) {
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub) {  // two 32-key sub-tiles
+    const int sk = sub * 32;
+    // st[e] = score of (key sk + 8*(e/4) + 4*lhalf + e%4, query lrow), seeded with mask/scale
+    floatx16 st;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const float4 mv = *reinterpret_cast<const float4*>(mk + sk + 8 * g + 4 * lhalf);
+      st[4 * g] = mv.x, st[4 * g + 1] = mv.y, st[4 * g + 2] = mv.z, st[4 * g + 3] = mv.w;
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const Chunk16 kf = *reinterpret_cast<const Chunk16*>(kt + sk * 128 + k_off[kk]);
+      st = mma16<T>(kf, qf[kk], st);
+    }
+    float mx = st[0];
+#pragma unroll
+    for (int e = 1; e < 16; ++e) mx = fmaxf(mx, st[e]);
+    {
+      // the other half-wavefront holds the remaining 16 keys of this query: exchange through
+      // v_permlane32_swap (two VALU instructions) instead of an LDS permute and its wait
+      const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, mx), __builtin_bit_cast(unsigned, mx), false, false);
+      mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+    }
+    // Lazy running maximum: the reference point m_run only moves when some query of the
+    // wavefront would otherwise see exp2 arguments above kSlack (fp16: probabilities up to 2^kSlack are
+    // as precise as smaller ones and the final division by the row sum cancels the choice of
+    // m_run), so the rescaling of the 32 output accumulators is skipped for most tiles.
+    if (__any((mx - m_run) * scale_log2e > kSlack<T>)) {
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) ot[t][e] *= alpha;
+    }
+    const float neg_m = -m_run * scale_log2e;
+    Chunk16 pf[2];
+    float psum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[2 * w], scale_log2e, neg_m));
+      const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[2 * w + 1], scale_log2e, neg_m));
+      const uint32_t pk = pack2<T>(p0, p1);
+      pf[w >> 2].w[w & 3] = pk;
+      psum = add_pair<T>(pk, psum);
+    }
+    l_run += psum;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const Chunk16 vf = *reinterpret_cast<const Chunk16*>(vt + t * 32 * 128 + k_off[2 * sub + kk]);
+        ot[t] = mma16<T>(vf, pf[kk], ot[t]);
+      }
+  }
+}
+
+// Normalise a wavefront's 32 x 64 output block and write it: ot[t][e] = O[query lrow][d = 32t + 8*(e/4) + 4*lhalf + e%4].
+// The block is staged in LDS (stage_base: the workgroup's LDS, free by now; 32 x (64 + 8) elements per wavefront) so
+// that it leaves as 128-byte rows.  out_head: first element of the head's columns in row 0 of this sequence.
+template <typename T>
+__device__ __forceinline__ void store_context(char* stage_base, int wave, int lane, const floatx16 (&ot)[2], float l_run,
+                                              T* out_head, int row_pitch, int q0, int q_end) {
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
+  const float inv = 1.0f / l_tot;
+  T* stage_o = reinterpret_cast<T*>(stage_base) + wave * (32 * (kD + 8));
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      Chunk8 c;
+      c.w[0] = pack2<T>(ot[t][4 * g] * inv, ot[t][4 * g + 1] * inv);
+      c.w[1] = pack2<T>(ot[t][4 * g + 2] * inv, ot[t][4 * g + 3] * inv);
+      *reinterpret_cast<Chunk8*>(stage_o + lrow * (kD + 8) + t * 32 + 8 * g + 4 * lhalf) = c;
+    }
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int r = p * 8 + (lane >> 3), cchunk = lane & 7;
+    const int qi = q0 + r;
+    if (qi < q_end) {
+      const Chunk16 x = *reinterpret_cast<const Chunk16*>(stage_o + r * (kD + 8) + cchunk * 8);
+      *reinterpret_cast<Chunk16*>(out_head + (int64_t)qi * row_pitch + cchunk * 8) = x;
+    }
+  }
+}
+
 template <typename T, bool PACKED, bool VT, int NW>
 __global__ __launch_bounds__(NW * 64, 16 / NW) void fused_attention_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                                  const T* __restrict__ v, const float* __restrict__ mask,
@@ -227,75 +325,16 @@ __global__ __launch_bounds__(NW * 64, 16 / NW) void fused_attention_kernel(const
   };
 
   // One 64-key tile from LDS stage STAGE (a compile-time constant so every LDS address is a
-  // per-lane base plus an immediate).  m_run is kept in raw score units; the softmax scale and
-  // log2(e) are applied inside the exp2 argument: p = exp2(s*c - m*c), c = scale*log2(e).
+  // per-lane base plus an immediate).
   const int k_lane = lrow * 128, k_sw = (lrow >> 1) & 7;
   int k_off[4];
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) k_off[kk] = k_lane + (((2 * kk + lhalf) ^ k_sw) << 4);  // rows +32 keep the swizzle
   auto compute_tile = [&](auto stage_c) {
     constexpr int STAGE = decltype(stage_c)::value;
-    const char* kt = smem + STAGE * kKBytes;
-    const char* vt = smem + 2 * kKBytes + STAGE * kVtBytes;
-    const float* mk = reinterpret_cast<const float*>(smem + 2 * kKBytes + 2 * kVtBytes) + STAGE * kBKV;
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {  // two 32-key sub-tiles
-      const int sk = sub * 32;
-      // st[e] = score of (key sk + 8*(e/4) + 4*lhalf + e%4, query lrow), seeded with mask/scale
-      floatx16 st;
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const float4 mv = *reinterpret_cast<const float4*>(mk + sk + 8 * g + 4 * lhalf);
-        st[4 * g] = mv.x, st[4 * g + 1] = mv.y, st[4 * g + 2] = mv.z, st[4 * g + 3] = mv.w;
-      }
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const Chunk16 kf = *reinterpret_cast<const Chunk16*>(kt + sk * 128 + k_off[kk]);
-        st = mma16<T>(kf, qf[kk], st);
-      }
-      float mx = st[0];
-#pragma unroll
-      for (int e = 1; e < 16; ++e) mx = fmaxf(mx, st[e]);
-      {
-        // the other half-wavefront holds the remaining 16 keys of this query: exchange through
-        // v_permlane32_swap (two VALU instructions) instead of an LDS permute and its wait
-        const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, mx), __builtin_bit_cast(unsigned, mx), false, false);
-        mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
-      }
-      // Lazy running maximum: the reference point m_run only moves when some query of the
-      // wavefront would otherwise see exp2 arguments above kSlack (fp16: probabilities up to 2^kSlack are
-      // as precise as smaller ones and the final division by the row sum cancels the choice of
-      // m_run), so the rescaling of the 32 output accumulators is skipped for most tiles.
-      if (__any((mx - m_run) * scale_log2e > kSlack<T>)) {
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
-        m_run = m_new;
-        l_run *= alpha;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) ot[t][e] *= alpha;
-      }
-      const float neg_m = -m_run * scale_log2e;
-      Chunk16 pf[2];
-      float psum = 0.f;
-#pragma unroll
-      for (int w = 0; w < 8; ++w) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[2 * w], scale_log2e, neg_m));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[2 * w + 1], scale_log2e, neg_m));
-        const uint32_t pk = pack2<T>(p0, p1);
-        pf[w >> 2].w[w & 3] = pk;
-        psum = add_pair<T>(pk, psum);
-      }
-      l_run += psum;
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const Chunk16 vf = *reinterpret_cast<const Chunk16*>(vt + t * 32 * 128 + k_off[2 * sub + kk]);
-          ot[t] = mma16<T>(vf, pf[kk], ot[t]);
-        }
-    }
+    attention_tile<T>(smem + STAGE * kKBytes, smem + 2 * kKBytes + STAGE * kVtBytes,
+                      reinterpret_cast<const float*>(smem + 2 * kKBytes + 2 * kVtBytes) + STAGE * kBKV, qf, k_off, lhalf,
+                      scale_log2e, ot, m_run, l_run);
   };
 
   const int tiles = (kv_len + kBKV - 1) / kBKV;
@@ -315,30 +354,8 @@ __global__ __launch_bounds__(NW * 64, 16 / NW) void fused_attention_kernel(const
     __syncthreads();
   }
 
-  // normalise and write: ot[t][e] = O[query lrow][d = 32t + 8*(e/4) + 4*lhalf + e%4]
-  const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
-  const float inv = 1.0f / l_tot;
-  // stage the wavefront's 32x64 tile in LDS (K buffers are free now) to store 128-byte rows
-  T* stage_o = reinterpret_cast<T*>(smem) + wave * (32 * (kD + 8));
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      Chunk8 c;
-      c.w[0] = pack2<T>(ot[t][4 * g] * inv, ot[t][4 * g + 1] * inv);
-      c.w[1] = pack2<T>(ot[t][4 * g + 2] * inv, ot[t][4 * g + 3] * inv);
-      *reinterpret_cast<Chunk8*>(stage_o + lrow * (kD + 8) + t * 32 + 8 * g + 4 * lhalf) = c;
-    }
-  const int hd = heads * kD;
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const int r = p * 8 + (lane >> 3), cchunk = lane & 7;
-    const int qi = q0 + r;
-    if (qi < q_len && qi < seq) {
-      const Chunk16 x = *reinterpret_cast<const Chunk16*>(stage_o + r * (kD + 8) + cchunk * 8);
-      *reinterpret_cast<Chunk16*>(out + ((int64_t)(out_row0 + qi)) * hd + head * kD + cchunk * 8) = x;
-    }
-  }
+  store_context<T>(smem, wave, lane, ot, l_run, out + (int64_t)out_row0 * (heads * kD) + head * kD, heads * kD, q0,
+                   min(q_len, seq));
 }
 
 }  // namespace ttmi

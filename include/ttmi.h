@@ -165,7 +165,10 @@ TTMI_API int ttmi_gemm_bias_layer_norm(const void* a, const void* w, void* out, 
  * allocates on first use.  The call reaches no hipMalloc / hipFree.  A problem whose K slices need more than
  * that buffer (slices * m * n * 4 bytes; the largest the encoder configurations produce is m = 2560, n = 768,
  * k = 3072 in three slices, 23.6 MB) is refused with TTMI_EINVAL; problems large enough to run unsplit need no
- * scratch and are accepted at any size.  The first call on a device resolves the buffer's address and sets kernel
+ * scratch and are accepted at any size.  One exception to "the same kernels": a product of a few thousand rows that
+ * ttmi_gemm_bias_layer_norm cuts in two on its large-tile kernel (an optimisation of a product that also runs whole;
+ * 6275 x 768 x 3072 is one) is cut here only if its partial products fit the buffer, and runs whole otherwise, with
+ * the 16-bit rounding of the product in front of the LayerNorm that large problems have.  The first call on a device resolves the buffer's address and sets kernel
  * attributes, so make one call outside a graph capture before capturing calls.  Nothing has to be cleared between calls (every partial tile that is read
  * has been written by the same call), but all calls on one GPU share the buffer: calls that overlap in time
  * on one GPU (different streams or threads) race. */

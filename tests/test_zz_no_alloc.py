@@ -63,6 +63,33 @@ def test_static_scratch_unsplit_problems_need_no_scratch(ttmi):
     _both(ttmi, "bf16", 8192, 1024, 1024, seed=10, fp32_residual=True)
 
 
+def test_static_scratch_and_the_two_slices_of_the_large_tile_kernel(ttmi):
+    """A product of a few thousand rows that the allocating entry point cuts in two on its large-tile kernel: where the
+    two fp32 partial products fit the static buffer (5000 x 768: 30.7 MB) both entry points run the same kernels and
+    agree bit for bit; where they do not (6275 x 768: 38.6 MB) the static form is not refused but runs the product
+    whole, so the two differ by the rounding of the 16-bit product in front of the LayerNorm and no more."""
+    ok(ttmi.ttmi_set_kernel_switch(b"TTMI_W4_SPLITK", 2))  # by itself the library takes two slices from about 5700 rows on
+    try:
+        _both(ttmi, "f16", 5000, 768, 3072, seed=11)
+    finally:
+        ok(ttmi.ttmi_set_kernel_switch(b"TTMI_W4_SPLITK", -1))
+    M, N, K = 6275, 768, 3072
+    rng = np.random.default_rng(12)
+    dA = dev(rng.standard_normal((M, K)).astype(np.float32), "f16")
+    dW = dev((rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32), "f16")
+    dres = dev(rng.standard_normal((M, N)).astype(np.float32), "f16")
+    bias, gamma, beta = (dev(rng.standard_normal(N).astype(np.float32), "f16") for _ in range(3))
+    outs = []
+    for fn in (ttmi.ttmi_gemm_bias_layer_norm, ttmi.ttmi_gemm_bias_layer_norm_static):
+        out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        ok(fn(ptr(dA), ptr(dW), ptr(out), ptr(dres), None, ptr(bias), ptr(gamma), ptr(beta), None, M, N, K, 1e-12,
+              TTMI_DTYPES["f16"], stream()))
+        outs.append(out)
+    torch.cuda.synchronize()
+    assert not torch.isnan(outs[1]).any()
+    assert float((outs[0].float() - outs[1].float()).abs().max()) < 2e-2
+
+
 def test_static_scratch_refuses_what_does_not_fit(ttmi):
     """With the admitted size lowered to 1 MiB the K slices of 2560 x 768 x 3072 (23.6 MB of partial tiles) no longer
     fit: the call is refused with TTMI_EINVAL and a message that names both sizes, nothing is launched and `out`

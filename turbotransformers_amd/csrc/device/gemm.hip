@@ -62,6 +62,12 @@ static int gemm_bias_layer_norm_impl(const void* a, const void* w, void* out, co
     int large_tile_slices = 0;
     if constexpr (sizeof(T) == 2) {
       if (rows_ok) large_tile_slices = w4_splitk_slices<T>(g, aligned);
+      // These slices are an optimisation of a product that also runs whole.  Where the caller has fixed the
+      // workspace (the static entry point) and the partial products do not fit it, the product runs whole instead of
+      // being refused.
+      if (large_tile_slices > 1 && tl_fixed_workspace.ptr != nullptr &&
+          (size_t)large_tile_slices * (size_t)m * (size_t)n * sizeof(float) > tl_fixed_workspace.bytes)
+        large_tile_slices = 0;
     }
     if (plan.kind != SplitKind::kNone || large_tile_slices > 1) {
       auto reduce = [&](const float* ws, int slices, bool, hipStream_t st) {

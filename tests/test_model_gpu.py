@@ -201,6 +201,37 @@ def test_golden_fixture_through_the_gpu_path(tt):
     assert max_abs(host(attn0), gold["attn.0"]) < 1e-5
 
 
+@pytest.mark.parametrize("dtype,B,S", [(torch.float16, 1, 128), (torch.float32, 2, 40), (torch.bfloat16, 3, 64)])
+def test_forward_replays_from_a_hip_graph(tt, dtype, B, S):
+    """In the steady state a forward allocates nothing, synchronises nothing and clears memory with kernels only, so
+    it can be captured into a HIP graph (launch-bound serving loops: one short sequence is 84 launches).  After a
+    warm-up on the capture stream (which sizes every buffer and the split-K workspace) the forward is captured once and
+    replayed three times, each replay on NEW ids written into the captured input tensor, with eager forwards of
+    other shapes in between; every replay must equal the eager forward of the same ids bit for bit."""
+    model, cfg = _hf_bert(2, seed=S)
+    tmodel = tt.BertModel.from_torch(model.to(dtype), torch.device("cuda:0"), "turbo")
+    gen = torch.Generator().manual_seed(S)
+    ids = torch.randint(0, cfg.vocab_size, (B, S), generator=gen).cuda()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            tmodel(ids)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        captured = tmodel(ids)[0]
+    for step in range(3):
+        fresh = torch.randint(0, cfg.vocab_size, (B, S), generator=gen).cuda()
+        want = tmodel(fresh)[0].clone()                                   # eager, same shape
+        tmodel(torch.randint(0, cfg.vocab_size, (B + 1, S + 8), generator=gen).cuda())  # eager, another shape
+        torch.cuda.synchronize()
+        ids.copy_(fresh)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, want), "replay %d" % step
+
+
 @pytest.mark.parametrize("lens", [[4, 1], [9, 7, 13], [10, 19, 20], [50, 3, 17, 31, 8]])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_smart_batch_equals_per_request_dense(tt, lens, dtype):

@@ -572,6 +572,40 @@ def run_ffn2_probe(iters=20, batch=64, seq=512, hidden=768, ffn=3072):
     print("\n".join(out_lines))
 
 
+def run_pmc_gemm(spec):
+    """Counter-collection helper: one bare product, `which,M,N,K,dtype` with which = ttmi (this library's ttmi_gemm) or
+    blaslt (torch.nn.functional.linear = hipBLASLt), on N(0,1) activations and N(0,0.02^2) weights; three warm-up and ten
+    timed launches, one line of text.  Run under `rocprofv3 --pmc ...` it puts the same counters on both kernels."""
+    import torch
+    from turbotransformers_amd import capi
+    which, m, n, k, dt = spec.split(",")
+    m, n, k = int(m), int(n), int(k)
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16}[dt]
+    cdt = {"f16": capi.F16, "bf16": capi.BF16}[dt]
+    torch.manual_seed(0)
+    a = torch.randn(m, k, device="cuda").to(tdt)
+    w = (torch.randn(n, k, device="cuda") * 0.02).to(tdt)
+    out = torch.empty(m, n, device="cuda", dtype=tdt)
+    if which == "ttmi":
+        lib = capi.load()
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+        fn = lambda: capi.check(lib.ttmi_gemm(P(a), P(w), P(out), m, n, k, k, k, n, 1, 1.0, 0.0, cdt,
+                                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    else:
+        fn = lambda: torch.nn.functional.linear(a, w)
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / 10 * 1e3
+    print("%s %d x %d x %d %s: %.1f us per launch, %.0f TFLOP/s" % (which, m, n, k, dt, us, 2.0 * m * n * k / us / 1e6))
+
+
 def cpu_baseline(seqs=4, seq=512, repeats=2):
     """The CPU oracle (an in-repo restatement of the reference's CPU branch: OpenMP loops + cblas_sgemm)
     on a bounded sample of the headline workload: `seqs` of the 64 sequences, all 12 layers, fp32; timed with 4 and
@@ -639,6 +673,9 @@ def main():
     ap.add_argument("--pmc-kernel", default=None,
                     help="counter-collection helper: run one calibration copy and a few launches of the named kernel "
                          "of the roofline pass (e.g. ffn1_gemm+bias+gelu), print nothing, exit")
+    ap.add_argument("--pmc-gemm", default=None, metavar="WHICH,M,N,K,DTYPE",
+                    help="counter-collection helper: a few launches of one bare product by this library (ttmi) or by "
+                         "hipBLASLt (blaslt), e.g. ttmi,32768,1024,4096,bf16; prints its time, exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (requests are independent; there is no multi-GPU step to time); "
@@ -652,6 +689,9 @@ def main():
     layers, hidden, heads, ffn, dtype, batch, seq = WORKLOADS[args.workload]
     if args.pmc_kernel:
         kernel_rooflines(dtype, batch, seq, hidden, heads, ffn, iters=3, only=args.pmc_kernel)
+        return
+    if args.pmc_gemm:
+        run_pmc_gemm(args.pmc_gemm)
         return
     if args.grid:
         print(json.dumps(run_grid(args.grid, args.steps, args.warmup)))

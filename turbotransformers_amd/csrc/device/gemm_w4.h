@@ -252,7 +252,8 @@ constexpr int w4_lds_bytes() {
 // BERT-base forward there, level at 192 wide), where the freed LDS also makes room for the third A stage.
 template <typename T, int BN, int MF, typename Epi, int AS = 2, bool DIRECT = false>
 __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, const Epi epi) {
-  static_assert(!DIRECT || (LinearDest<Epi>::value && MF == 16), "direct stores: row-major 16-bit outputs, 16-wide blocks");
+  static_assert(!DIRECT || ((LinearDest<Epi>::value || HasColumnPass<Epi>::value) && MF == 16),
+                "direct stores: row-major 16-bit outputs or the head split, 16-wide blocks");
   static_assert(sizeof(T) == 2, "16-bit operands");
   static_assert(MF == 32 || MF == 16, "block sizes of the matrix instructions");
   static_assert(AS == 2 || (AS == 3 && MF == 16 && !HasColumnPass<Epi>::value), "three A stages: 16-wide blocks, row-major epilogues");
@@ -368,7 +369,17 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
   auto store_c = [&](Quad x, uint32_t voff, uint32_t soff) __attribute__((always_inline)) {
     __builtin_amdgcn_raw_buffer_store_b128(x, rsrc_c, (int)voff, (int)soff, 0);
   };
+  // direct stores of the head split: one resource per destination tensor, each [B, heads, S, d] = M x hidden elements
+  // (the launcher checks that this is below 2 GiB and that 16 consecutive rows share a sequence)
+  auto head_split_store = [&](Quad x, int which, uint32_t voff, uint32_t soff) __attribute__((always_inline)) {
+    if constexpr (DIRECT && HasColumnPass<Epi>::value) {
+      T* base = which == 0 ? epi.q : (which == 1 ? epi.k : epi.v);
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)((int64_t)g.m * epi.hidden * (int64_t)sizeof(T)), 0x00020000);
+      __builtin_amdgcn_raw_buffer_store_b128(x, rsrc, (int)voff, (int)soff, 0);
+    }
+  };
 #else
+  auto head_split_store = [&](Quad, int, uint32_t, uint32_t) {};
   auto dma_issue_one = [&](int) {};
   const uint32_t ldc_bytes = 0;
   auto store_c = [&](Quad, uint32_t, uint32_t) {};
@@ -700,7 +711,7 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       // epilogues that scatter (the QKV split): the column part of a lane's destinations, once per tile
       T* col_ptr[PASSES];
       bool block_in_one_sequence = false;  // uniform: the rows of a group share their batch index
-      if constexpr (!LinearDest<Epi>::value && !StoresF32<Epi>::value) {
+      if constexpr (!LinearDest<Epi>::value && !StoresF32<Epi>::value && !DIRECT) {
         block_in_one_sequence = epi.rows_share_sequence(GROUP);
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
@@ -710,6 +721,9 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
       }
       // direct stores: row lrow of a 16-row block, the lane's 16 bytes of a 64-byte run (unit_chunk(0) names them)
       const uint32_t direct_voff = (uint32_t)lrow * ldc_bytes + (uint32_t)unit_chunk(0) * 16u;
+      uint32_t head_split_voff = 0;  // the same for the head split: rows of a head are `dim` elements apart
+      if constexpr (DIRECT && HasColumnPass<Epi>::value)
+        head_split_voff = (uint32_t)lrow * (uint32_t)epi.dim * (uint32_t)sizeof(T) + (uint32_t)unit_chunk(0) * 16u;
       Quad landed[PASSES];  // first-class vectors: arrays of a struct type may end up in scratch memory
       // The matrix instructions are inline asm, so the compiler's hazard recogniser does not see that the accumulator
       // reads below depend on them: wait out the longest write-to-read distance of the matrix pipe here.
@@ -764,9 +778,23 @@ __global__ __launch_bounds__(kW4Threads) void gemm_w4_kernel(const GemmArgs g, c
                 // 16-row block goes into the scalar offset, the pair of block columns into the immediate
                 const int rblk = i * GROUP + 16 * (v / (CB / 2));  // first row of the unit's 16-row block inside the wavefront's 128
                 const int ncol = wn0 + unit_chunk(v) * 8;
-                if ((whole_rows || m0 + wm0 + rblk + lrow < m_lim) && (whole_width || n0 + ncol < n_lim))
-                  store_c(packed[v], direct_voff + (uint32_t)(v % (CB / 2)) * 64u,
-                          (uint32_t)(m0 + wm0 + rblk) * ldc_bytes + (uint32_t)(n0 + wn0) * (uint32_t)sizeof(T));
+                if constexpr (LinearDest<Epi>::value) {
+                  if ((whole_rows || m0 + wm0 + rblk + lrow < m_lim) && (whole_width || n0 + ncol < n_lim))
+                    store_c(packed[v], direct_voff + (uint32_t)(v % (CB / 2)) * 64u,
+                            (uint32_t)(m0 + wm0 + rblk) * ldc_bytes + (uint32_t)(n0 + wn0) * (uint32_t)sizeof(T));
+                } else if constexpr (HasColumnPass<Epi>::value) {
+                  // Head split: the unit's 32 columns lie in one head of one of q, k, v and its 16 rows in one
+                  // sequence (both uniform), so the destination is a scalar offset plus the lane's row and column
+                  // share: element ((b * heads + head) * seq + s) * dim + i of that tensor.
+                  const uint32_t c32 = (uint32_t)(n0 + wn0 + 32 * (v % (CB / 2)));  // first of the unit's 32 columns
+                  const uint32_t which = epi.div_hidden.div(c32), rem = c32 - which * (uint32_t)epi.hidden;
+                  const uint32_t head = epi.div_dim.div(rem), i0 = rem - head * (uint32_t)epi.dim;
+                  const uint32_t r16 = (uint32_t)(m0 + wm0 + rblk);                 // first of the unit's 16 rows
+                  const uint32_t b = epi.div_seq.div(min(r16, (uint32_t)m_lim - 1u)), s16 = r16 - b * (uint32_t)epi.seq;
+                  const uint32_t soff = (((b * (uint32_t)epi.heads + head) * (uint32_t)epi.seq + s16) * (uint32_t)epi.dim + i0) * (uint32_t)sizeof(T);
+                  if ((whole_rows || m0 + wm0 + rblk + lrow < m_lim) && (whole_width || n0 + ncol < n_lim))
+                    head_split_store(packed[v], (int)which, head_split_voff, soff);
+                }
               }
             }
           }
@@ -949,7 +977,8 @@ static int launch_w4(GemmArgs g, const Epi& epi, hipStream_t s, int split_col = 
     if (kernel_switch(kSwitchW4AStages) != 2) return launch_w4<T, BN, Epi, 3, true>(g, epi, s, split_col);
     return launch_w4<T, BN, Epi, 2, true>(g, epi, s, split_col);
   }
-  constexpr int LDS = w4_lds_bytes<BN, kW4Block, AS, DIRECT || StoresF32<Epi>::value>();
+  // (the head split keeps its strips with direct stores too: its transposed-V tiles leave through them)
+  constexpr int LDS = w4_lds_bytes<BN, kW4Block, AS, (DIRECT && !HasColumnPass<Epi>::value) || StoresF32<Epi>::value>();
   static_assert(LDS <= kLdsPerCu, "tile does not fit in LDS");
   const int slices = g.k_chunk > 0 ? g.k / g.k_chunk : 1;  // K slices: fp32 outputs only (launch_w4_splitk)
   if (describe_only(AS == 3 ? "dma3_agpr" : "dma_agpr", 4, 256, BN, slices)) return 0;
@@ -1086,9 +1115,18 @@ struct LargeTileKernel<T, EpiQkvSplit<T, false>, typename std::enable_if<sizeof(
     (void)pick_tile(g.m, g.n, batch, &other);
     return cost(g, epi, batch) < other;
   }
+  // Q, K (and a row-major V) leave straight from the accumulator layout when every 16-row block lies in one sequence and
+  // every 32-column group in one head, and a destination tensor stays below 2 GiB (32-bit buffer offsets).
+  static bool direct_ok(const GemmArgs& g, const Epi& epi) {
+    return epi.seq % 16 == 0 && epi.dim % 32 == 0 && g.m % epi.seq == 0 && g.n == 3 * epi.hidden &&
+           (int64_t)g.m * epi.hidden * (int64_t)sizeof(T) < ((int64_t)1 << 31);
+  }
   static int launch(const GemmArgs& g, const Epi& epi, hipStream_t s) {
-    if (fits256(g, epi) && tile_cost(kTile256, g.m, g.n, 1) < cost192(g, epi, 1)) return launch_w4<T, 256>(g, epi, s);
-    return launch_w4<T, 192>(g, epi, s, split_run(g, epi) ? 2 * epi.hidden : 0);
+    const bool direct = direct_ok(g, epi);
+    if (fits256(g, epi) && tile_cost(kTile256, g.m, g.n, 1) < cost192(g, epi, 1))
+      return direct ? launch_w4<T, 256, Epi, 2, true>(g, epi, s) : launch_w4<T, 256>(g, epi, s);
+    const int split_col = split_run(g, epi) ? 2 * epi.hidden : 0;
+    return direct ? launch_w4<T, 192, Epi, 2, true>(g, epi, s, split_col) : launch_w4<T, 192>(g, epi, s, split_col);
   }
 };
 // fp32 output of a 16-bit product (the projections in front of a LayerNorm in bfloat16 models).
